@@ -8,9 +8,11 @@ from . import pelalix  # registers Pelalix
 from .pelalix import PelalixConfig
 from . import dezudra  # registers Dezudra
 from .dezudra import DezudraConfig
+from . import bibevik  # registers Bibevik
+from .bibevik import BibevikConfig
 
 __all__ = [
     "ConfigError", "config_class_for", "config_from_dict", "config_from_directory", "config_from_json",
     "known_architectures", "register_architecture", "LayerSpec", "ModelSpec", "PartSpec", "ScheduleEntry", "linear_head", "token_embedding",
-    "Qwen2MoeConfig", "PelalixConfig", "DezudraConfig",
+    "Qwen2MoeConfig", "PelalixConfig", "DezudraConfig", "BibevikConfig",
 ]

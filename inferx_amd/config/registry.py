@@ -63,4 +63,16 @@ def config_from_directory(model_dir: str):
     if not os.path.isfile(path):
         raise ConfigError(f"{path}: no such file")
     with open(path, "r", encoding="utf-8") as f:
-        return config_from_json(f.read())
+        cfg = config_from_json(f.read())
+    resolve = getattr(cfg, "resolve_shapes", None)
+    if resolve is not None:
+        # a design may leave sizes to the shapes of its tensors: the checkpoint's header is read for them
+        from ..weights.safetensors_io import Checkpoint, CheckpointError
+        try:
+            ckpt = Checkpoint.open(model_dir)
+        except (CheckpointError, OSError):
+            ckpt = None
+        if ckpt is not None:
+            resolve({name: tuple(ckpt.shape(name)) for name in ckpt.names()})
+            cfg.validate()
+    return cfg

@@ -120,6 +120,26 @@ __device__ __forceinline__ float ix_block_max(float v, float* red) {
   return total;
 }
 
+// What a gated product makes of its two sums g and u.  limit <= 0: silu(g) * u.  limit > 0, the clamped form:
+// g = min(g, limit), u = clamp(u, -limit, limit), then g * sigmoid(1.702 g) * (u + 1).
+#define IX_GLU_ALPHA 1.702f
+template <bool FAST = false>
+__device__ __forceinline__ float ix_glu(float g, float u, float limit) {
+  float steep = 1.0f;
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit) + 1.0f;
+    steep = IX_GLU_ALPHA;
+  }
+  const float e = FAST ? __expf(-steep * g) : expf(-steep * g);
+  return g / (1.0f + e) * u;
+}
+
+// bits of a router's selection mode
+#define IX_ROUTE_RENORMALIZE 1  // the chosen weights are divided by their sum
+#define IX_ROUTE_SIGMOID 2      // an expert's score is sigmoid(z) of its own logit instead of the softmax over all
+#define IX_ROUTE_GROUP_TOP2 4   // a group's score is the sum of its two best scores instead of its best
+
 // ---- host side -------------------------------------------------------------
 #include <algorithm>
 #include <string>

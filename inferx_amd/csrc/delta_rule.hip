@@ -399,13 +399,15 @@ extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dt
 //
 //   o = x - lambda x2  (x2 optional);  y = o / sqrt(mean(o^2) + eps) * weight (optional) * silu(gate) (optional) * mult
 //
-// x, x2 float32 [T, heads, vdim]; weight [vdim], shared by the heads; gate of the run's type at
+// x, x2 float32 [T, heads, vdim]; weight [vdim], shared by the heads (or [heads, vdim] with `weight_per_head`);
+// `gate_sigmoid`: sigmoid(gate) instead of silu(gate); gate of the run's type at
 // gate[t * gate_stride + head * vdim + j]; out of the run's type [T, heads * vdim].
 template <typename T>
 __global__ void __launch_bounds__(256)
 head_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ x2, float lambda,
                       const void* __restrict__ weight, int w_dtype, const T* __restrict__ gate, int64_t gate_stride,
-                      T* __restrict__ out, int64_t pairs, int heads, int vdim, float eps, float mult) {
+                      T* __restrict__ out, int64_t pairs, int heads, int vdim, float eps, float mult,
+                      int weight_per_head, int gate_sigmoid) {
   const int64_t p = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (p >= pairs) return;
   const int lane = threadIdx.x & 63;
@@ -422,10 +424,10 @@ head_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ x2,
   const float inv = mult / sqrtf(ss / static_cast<float>(vdim) + eps);
   for (int j = lane; j < vdim; j += 64) {
     float y = (x2r ? xr[j] - lambda * x2r[j] : xr[j]) * inv;
-    if (weight) y *= ix_load_rt(weight, w_dtype, j);
+    if (weight) y *= ix_load_rt(weight, w_dtype, weight_per_head ? head * vdim + j : j);
     if (gate) {
       const float gv = ix_load(gate + t * gate_stride + head * vdim + j);
-      y *= gv / (1.0f + expf(-gv));
+      y *= (gate_sigmoid ? 1.0f : gv) / (1.0f + expf(-gv));
     }
     ix_store(out + p * vdim + j, y);
   }
@@ -433,7 +435,8 @@ head_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ x2,
 
 extern "C" int ix_head_norm_gate(const float* x, const float* x2, float lambda, const void* weight, int w_dtype,
                                  const void* gate, int64_t gate_stride, void* out, int dtype, int64_t tokens,
-                                 int heads, int vdim, float eps, float mult, hipStream_t stream) {
+                                 int heads, int vdim, float eps, float mult, int weight_per_head, int gate_sigmoid,
+                                 hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && heads > 0 && vdim > 0, "sizes must be positive");
   IX_REQUIRE(dtype == IX_F32 || dtype == IX_BF16, "dtype must be float32 or bfloat16");
   if (tokens == 0) return 0;
@@ -442,9 +445,11 @@ extern "C" int ix_head_norm_gate(const float* x, const float* x2, float lambda, 
   dim3 grid(static_cast<unsigned>((pairs + 3) / 4)), block(256);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, x, x2, lambda, weight, w_dtype,
-                       (const float*)gate, gate_stride, (float*)out, pairs, heads, vdim, eps, mult);
+                       (const float*)gate, gate_stride, (float*)out, pairs, heads, vdim, eps, mult, weight_per_head,
+                       gate_sigmoid);
   else
     hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, stream, x, x2, lambda, weight, w_dtype,
-                       (const bf16_t*)gate, gate_stride, (bf16_t*)out, pairs, heads, vdim, eps, mult);
+                       (const bf16_t*)gate, gate_stride, (bf16_t*)out, pairs, heads, vdim, eps, mult, weight_per_head,
+                       gate_sigmoid);
   return ix_check_launch("ix_head_norm_gate");
 }

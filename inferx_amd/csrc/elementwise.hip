@@ -549,3 +549,72 @@ extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, 
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_qkv_rope_append");
 }
+
+// ---------------------------------------------------------------------------
+// out[t, i] = glu(gu[t, i] + bias[i], gu[t, width + i] + bias[width + i]) with `ix_glu` (silu(g) * u, or with a
+// limit the clamped form); the bias (2 * width numbers, gate's first) may be absent.
+template <typename T>
+__global__ void glu_bias_kernel(const T* __restrict__ gu, const void* __restrict__ bias, int bias_dtype,
+                                T* __restrict__ out, int64_t tokens, int64_t width, float limit) {
+  const int64_t n = tokens * width;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = i / width, c = i - t * width;
+    float g = ix_load(gu + t * 2 * width + c);
+    float u = ix_load(gu + t * 2 * width + width + c);
+    if (bias) {
+      g += ix_load_rt(bias, bias_dtype, c);
+      u += ix_load_rt(bias, bias_dtype, width + c);
+    }
+    ix_store(out + i, ix_glu(g, u, limit));
+  }
+}
+
+extern "C" int ix_glu_bias(const void* gu, const void* bias, int bias_dtype, void* out, int dtype, int64_t tokens,
+                           int64_t width, float limit, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  if (tokens == 0) return 0;
+  const int64_t n = tokens * width;
+  dim3 grid(static_cast<unsigned>(std::min<int64_t>((n + 255) / 256, 65536))), block(256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(glu_bias_kernel<float>, grid, block, 0, stream, (const float*)gu, bias, bias_dtype,
+                       (float*)out, tokens, width, limit);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(glu_bias_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, bias, bias_dtype,
+                       (bf16_t*)out, tokens, width, limit);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_glu_bias");
+}
+
+// ---------------------------------------------------------------------------
+// h[t, c] += a[t, c] + b[t, c] + bias[c]: two branches' results (the second and the bias may be absent) summed in
+// float32 and added to the float32 residual stream.
+template <typename T>
+__global__ void add_branches_kernel(float* __restrict__ h, const T* __restrict__ a, const T* __restrict__ b,
+                                    const void* __restrict__ bias, int bias_dtype, int64_t n, int64_t width) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    float d = ix_load(a + i);
+    if (b) d += ix_load(b + i);
+    if (bias) d += ix_load_rt(bias, bias_dtype, i % width);
+    h[i] += d;
+  }
+}
+
+extern "C" int ix_add_branches(float* h, const void* a, const void* b, int dtype, const void* bias, int bias_dtype,
+                               int64_t tokens, int64_t width, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  if (tokens == 0) return 0;
+  const int64_t n = tokens * width;
+  dim3 grid(static_cast<unsigned>(std::min<int64_t>((n + 255) / 256, 65536))), block(256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(add_branches_kernel<float>, grid, block, 0, stream, h, (const float*)a, (const float*)b, bias,
+                       bias_dtype, n, width);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(add_branches_kernel<bf16_t>, grid, block, 0, stream, h, (const bf16_t*)a, (const bf16_t*)b,
+                       bias, bias_dtype, n, width);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_add_branches");
+}

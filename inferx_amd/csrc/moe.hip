@@ -32,23 +32,29 @@ __device__ __forceinline__ void route_select(float* z, float* red, float* __rest
   float mx = -INFINITY;
   for (int e = tid; e < experts; e += blockDim.x) mx = fmaxf(mx, z[e]);
   mx = ix_block_max(mx, red);
+  const bool sigmoid = renormalize & IX_ROUTE_SIGMOID;  // (`renormalize` holds the selection mode's bits)
   float sum = 0.f;
   for (int e = tid; e < experts; e += blockDim.x) {
-    const float p = expf(z[e] - mx);
+    const float p = sigmoid ? 1.0f / (1.0f + expf(-z[e])) : expf(z[e] - mx);
     z[e] = p;
     sum += p;
   }
   sum = ix_block_sum(sum, red);  // its barriers also publish z
   if (wave != 0) return;
-  const float inv_sum = 1.0f / sum;
+  const float inv_sum = sigmoid ? 1.0f : 1.0f / sum;
   if (groups_keep < n_groups) {
     // The experts form n_groups equal groups of neighbours (at most 64), a group's score is its largest score, and
     // only experts of the groups_keep best groups can be chosen (among equal groups the lower number first): the
     // others' scores are struck out before the rounds below.  The weights stay the scores over all experts.
     const int per = experts / n_groups;
-    float best = -INFINITY;
+    float best = -INFINITY, second = -INFINITY;
     if (lane < n_groups)
-      for (int e = lane * per; e < (lane + 1) * per; ++e) best = fmaxf(best, z[e]);
+      for (int e = lane * per; e < (lane + 1) * per; ++e) {
+        const float v = z[e];
+        if (v > best) { second = best; best = v; }
+        else if (v > second) second = v;
+      }
+    if ((renormalize & IX_ROUTE_GROUP_TOP2) && per > 1) best += second;  // (or the sum of its two largest)
     bool kept = false;
     for (int round = 0; round < groups_keep; ++round) {
       float bv = best;
@@ -85,7 +91,7 @@ __device__ __forceinline__ void route_select(float* z, float* red, float* __rest
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
   }
-  const float f = ((renormalize && total > 0.f) ? 1.0f / total : 1.0f) * scale;
+  const float f = (((renormalize & IX_ROUTE_RENORMALIZE) && total > 0.f) ? 1.0f / total : 1.0f) * scale;
   if (lane < k) topk_w[t * (k + always) + lane] = chosen * f;
   if (lane < always) {
     topk_e[t * (k + always) + k + lane] = experts + lane;
@@ -400,7 +406,7 @@ template <typename TA, typename TW, typename TO, bool GATE_UP>
 __global__ void __launch_bounds__(256)
 moe_grouped_plain_kernel(const TA* __restrict__ a, const TW* __restrict__ w, TO* __restrict__ out,
                          const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows, int experts,
-                         int64_t n_out, int64_t width, int act) {
+                         int64_t n_out, int64_t width, int act, float glu_limit) {
   __shared__ float As[GG_BK][GG_BM + 4];
   __shared__ float Ws[GATE_UP ? 2 : 1][GG_BK][GG_BN + 4];
   __shared__ int32_t src_row[GG_BM];
@@ -476,7 +482,7 @@ moe_grouped_plain_kernel(const TA* __restrict__ a, const TW* __restrict__ w, TO*
       const int64_t n = n0 + tx * 4 + j;
       if (n >= n_out) continue;
       float v = acc[0][i][j];
-      if (GATE_UP) v = v / (1.0f + expf(-v)) * acc[1][i][j];
+      if (GATE_UP) v = ix_glu(v, acc[1][i][j], glu_limit);
       else if (act) v = v > 0.f ? v * v : 0.f;  // the square of relu
       ix_store(out + static_cast<int64_t>(r) * n_out + n, v);
     }
@@ -486,12 +492,12 @@ moe_grouped_plain_kernel(const TA* __restrict__ a, const TW* __restrict__ w, TO*
 template <bool GATE_UP>
 static int launch_grouped_plain(const void* a, int a_dtype, const void* w, int w_dtype, void* out,
                                 const int32_t* offsets, const int32_t* rows, int64_t assignments, int experts,
-                                int64_t n_out, int64_t width, int act, hipStream_t stream) {
+                                int64_t n_out, int64_t width, int act, float glu_limit, hipStream_t stream) {
   const int64_t m_tiles = std::min<int64_t>(assignments, (assignments + GG_BM - 1) / GG_BM + experts);
   dim3 grid((n_out + GG_BN - 1) / GG_BN, m_tiles), block(256);
 #define LAUNCH(TA, TW)                                                                                            \
   hipLaunchKernelGGL((moe_grouped_plain_kernel<TA, TW, TA, GATE_UP>), grid, block, 0, stream, (const TA*)a,        \
-                     (const TW*)w, (TA*)out, offsets, rows, experts, n_out, width, act)
+                     (const TW*)w, (TA*)out, offsets, rows, experts, n_out, width, act, glu_limit)
   if (a_dtype == IX_F32 && w_dtype == IX_F32) LAUNCH(float, float);
   else if (a_dtype == IX_F32 && w_dtype == IX_BF16) LAUNCH(float, bf16_t);
   else if (a_dtype == IX_BF16 && w_dtype == IX_F32) LAUNCH(bf16_t, float);
@@ -503,15 +509,15 @@ static int launch_grouped_plain(const void* a, int a_dtype, const void* w, int w
 
 extern "C" int ix_moe_grouped_plain(const void* a, int a_dtype, const void* w, int w_dtype, void* out,
                                     const int32_t* offsets, const int32_t* rows, int64_t assignments, int experts,
-                                    int64_t n_out, int64_t width, int gate_up, hipStream_t stream) {
+                                    int64_t n_out, int64_t width, int gate_up, float glu_limit, hipStream_t stream) {
   IX_REQUIRE(assignments >= 0 && n_out > 0 && width > 0 && experts > 0, "sizes must be positive");
   IX_REQUIRE(assignments < (1ll << 31) / GG_BM, "too many assignments");
   if (assignments == 0) return 0;
   IX_REQUIRE(gate_up >= 0 && gate_up <= 2, "gate_up must be 0 (plain), 1 (gate|up with SwiGLU) or 2 (square of relu)");
   return gate_up == 1 ? launch_grouped_plain<true>(a, a_dtype, w, w_dtype, out, offsets, rows, assignments, experts,
-                                                   n_out, width, 0, stream)
+                                                   n_out, width, 0, glu_limit, stream)
                       : launch_grouped_plain<false>(a, a_dtype, w, w_dtype, out, offsets, rows, assignments, experts,
-                                                    n_out, width, gate_up == 2 ? 1 : 0, stream);
+                                                    n_out, width, gate_up == 2 ? 1 : 0, 0.f, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -32,7 +32,7 @@ template <int MT, bool GATE_UP, int KSPLIT, typename TO = __bf16, int NB = 1>
 __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
                                              TO* __restrict__ out, const int32_t* __restrict__ rows, int e,
                                              int row0, int row_end, int n0, int n_out, int width, float* red,
-                                             int act = 0) {
+                                             int act = 0, float glu_limit = 0.f) {
   constexpr int NACC = NB * (GATE_UP ? 2 : 1);  // accumulator b + NB h: block b of the gate (h = 0) or up (1) rows
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m = lane & 15, g = lane >> 4;
@@ -156,7 +156,7 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         v[i] = acc[u][t][i];
-        if constexpr (GATE_UP) v[i] = v[i] / (1.0f + __expf(-v[i])) * acc[NB + u][t][i];
+        if constexpr (GATE_UP) v[i] = ix_glu<true>(v[i], acc[NB + u][t][i], glu_limit);
         else if (act) v[i] = v[i] > 0.f ? v[i] * v[i] : 0.f;  // the square of relu
       }
       TO* dst = out + static_cast<int64_t>(r) * n_out + nb;
@@ -192,14 +192,14 @@ __global__ void __launch_bounds__(256)
 moe_grouped_mfma_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ out,
                         const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
                         const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
-                        const int32_t* __restrict__ tile_info, int n_out, int width, int act) {
+                        const int32_t* __restrict__ tile_info, int n_out, int width, int act, float glu_limit) {
   __shared__ float red[KSPLIT > 1 ? 3 * 64 * MT * (GATE_UP ? 2 : 1) * 4 : 1];
   if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
   const int e = tile_expert[blockIdx.y];
   const int n0 = (KSPLIT > 1 ? blockIdx.x : blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;
   if (n0 >= n_out) return;  // whole wavefront (KSPLIT == 1) or whole workgroup
   grouped_body<MT, GATE_UP, KSPLIT>(a, w, out, rows, e, tile_row0[blockIdx.y], offsets[e + 1], n0, n_out, width, red,
-                                    act);
+                                    act, glu_limit);
 }
 
 // Routed experts and the shared expert in one launch (decoding: every launch saved counts).  The first
@@ -213,7 +213,7 @@ moe_grouped_dual_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ o
                         const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
                         const int32_t* __restrict__ tile_info, int max_tiles, int n_out, int width,
                         const __bf16* a_s, const __bf16* w_s, __bf16* __restrict__ out_s,
-                        int shared_rows, int n_out_s, int width_s) {
+                        int shared_rows, int n_out_s, int width_s, float glu_limit, float glu_limit_s) {
   __shared__ float red[3 * 64 * MT * NB * (GATE_UP ? 2 : 1) * 4];
   const int n16_s = (n_out_s + 16 * NB - 1) / (16 * NB);  // column blocks of 16 NB out-features
   const int shared_blocks = n16_s * ((shared_rows + 16 * MT - 1) / (16 * MT));
@@ -222,7 +222,7 @@ moe_grouped_dual_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ o
     const int tile = idx / n16_s;
     grouped_body<MT, GATE_UP, 4, __bf16, NB>(a_s, w_s, out_s, nullptr, 0, tile * 16 * MT, shared_rows,
                                              (idx - tile * n16_s) * 16 * NB,
-                                 n_out_s, width_s, red);
+                                 n_out_s, width_s, red, 0, glu_limit_s);
   } else {
     idx -= shared_blocks;
     const int n16_e = (n_out + 16 * NB - 1) / (16 * NB);
@@ -230,17 +230,18 @@ moe_grouped_dual_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ o
     if (tile >= tile_info[0]) return;
     const int e = tile_expert[tile];
     grouped_body<MT, GATE_UP, 4, __bf16, NB>(a, w, out, rows, e, tile_row0[tile], offsets[e + 1],
-                                             (idx - tile * n16_e) * 16 * NB, n_out, width, red);
+                                             (idx - tile * n16_e) * 16 * NB, n_out, width, red, 0, glu_limit);
   }
 }
 
 // `max_tiles` bounds the number of row tiles (the grid); the kernel reads the true number from tile_info.
 // tile_rows (16, 32 or 64) must be what the grouping kernel was given.  gate_up: 0 a plain product, 1 gate|up rows
-// with SwiGLU, 2 a plain product whose results pass the square of relu.
+// with SwiGLU, 2 a plain product whose results pass the square of relu.  glu_limit > 0: the gate|up rows meet in
+// the clamped form (`ix_glu`).
 extern "C" int ix_moe_grouped_mfma(const void* a, const void* w, void* out, const int32_t* offsets,
                                    const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
                                    const int32_t* tile_info, int max_tiles, int tile_rows, int64_t n_out,
-                                   int64_t width, int gate_up, int k_split, hipStream_t stream) {
+                                   int64_t width, int gate_up, int k_split, float glu_limit, hipStream_t stream) {
   IX_REQUIRE(n_out > 0 && width > 0 && max_tiles >= 0, "sizes must be positive");
   IX_REQUIRE(width % 8 == 0, "the reduction width must be a multiple of 8 for the matrix-core kernel");
   IX_REQUIRE(n_out < (1 << 30) && width < (1 << 30), "sizes too large");
@@ -254,7 +255,7 @@ extern "C" int ix_moe_grouped_mfma(const void* a, const void* w, void* out, cons
 #define LAUNCH(MT, GU, KS)                                                                                        \
   hipLaunchKernelGGL((moe_grouped_mfma_kernel<MT, GU, KS>), grid, block, 0, stream, (const __bf16*)a,             \
                      (const __bf16*)w, (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, \
-                     (int)width, gate_up == 2 ? 1 : 0)
+                     (int)width, gate_up == 2 ? 1 : 0, glu_limit)
 #define PICK(MT)                                       \
   if (gate_up == 1) {                                  \
     if (k_split > 1) LAUNCH(MT, true, 4);              \
@@ -275,7 +276,8 @@ extern "C" int ix_moe_grouped_dual(const void* a, const void* w, void* out, cons
                                    const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
                                    const int32_t* tile_info, int max_tiles, int tile_rows, int64_t n_out,
                                    int64_t width, const void* a_s, const void* w_s, void* out_s, int shared_rows,
-                                   int64_t n_out_s, int64_t width_s, int gate_up, hipStream_t stream) {
+                                   int64_t n_out_s, int64_t width_s, int gate_up, float glu_limit, float glu_limit_s,
+                                   hipStream_t stream) {
   IX_REQUIRE(n_out > 0 && width > 0 && n_out_s > 0 && width_s > 0 && max_tiles >= 0 && shared_rows > 0,
              "sizes must be positive");
   IX_REQUIRE(width % 8 == 0 && width_s % 8 == 0, "the reduction widths must be multiples of 8");
@@ -293,7 +295,7 @@ extern "C" int ix_moe_grouped_dual(const void* a, const void* w, void* out, cons
   hipLaunchKernelGGL((moe_grouped_dual_kernel<MT, GU, NB>), grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w, \
                      (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, max_tiles, (int)n_out,        \
                      (int)width, (const __bf16*)a_s, (const __bf16*)w_s, (__bf16*)out_s, shared_rows, (int)n_out_s, \
-                     (int)width_s)
+                     (int)width_s, glu_limit, glu_limit_s)
 #define PICK(MT, NB)                 \
   if (gate_up == 1) LAUNCH(MT, true, NB); \
   else LAUNCH(MT, false, NB);

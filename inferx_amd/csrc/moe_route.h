@@ -105,23 +105,29 @@ select_dispatch_body(const float* logits, float* __restrict__ topk_w, int32_t* _
     }
     if (shared_gate && lane == 0) shared_gate[t] = 1.0f / (1.0f + expf(-fresh(row + experts)));
     mx = ix_wave_max(mx);
+    const bool sigmoid = renormalize & IX_ROUTE_SIGMOID;  // (`renormalize` holds the selection mode's bits)
     float sum = 0.f;
     for (int e = lane; e < experts; e += 64) {
-      const float p = expf(z[e] - mx);
+      const float p = sigmoid ? 1.0f / (1.0f + expf(-z[e])) : expf(z[e] - mx);
       z[e] = p;
       sum += p;
     }
     sum = ix_wave_sum(sum);
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
-    const float inv_sum = 1.0f / sum;
+    const float inv_sum = sigmoid ? 1.0f : 1.0f / sum;
     if (groups_keep < n_groups) {
       // equal groups of neighbouring experts (at most 64), scored by their best expert: the experts of all but the
       // groups_keep best groups (among equals the lower number first) are struck out before the rounds below
       const int per = experts / n_groups;
-      float best = -INFINITY;
+      float best = -INFINITY, second = -INFINITY;
       if (lane < n_groups)
-        for (int e = lane * per; e < (lane + 1) * per; ++e) best = fmaxf(best, z[e]);
+        for (int e = lane * per; e < (lane + 1) * per; ++e) {
+          const float v = z[e];
+          if (v > best) { second = best; best = v; }
+          else if (v > second) second = v;
+        }
+      if ((renormalize & IX_ROUTE_GROUP_TOP2) && per > 1) best += second;  // (or the sum of its two largest)
       bool kept = false;
       for (int round = 0; round < groups_keep; ++round) {
         float bv = best;
@@ -158,7 +164,7 @@ select_dispatch_body(const float* logits, float* __restrict__ topk_w, int32_t* _
       __builtin_amdgcn_wave_barrier();
       __threadfence_block();
     }
-    const float f = ((renormalize && total > 0.f) ? 1.0f / total : 1.0f) * scale;
+    const float f = (((renormalize & IX_ROUTE_RENORMALIZE) && total > 0.f) ? 1.0f / total : 1.0f) * scale;
     if (lane < k) topk_w[t * k + lane] = mine_w * f;
   }
   __syncthreads();
@@ -272,27 +278,42 @@ select_dispatch_few(const float* logits, float* __restrict__ topk_w, int32_t* __
     }
     if (shared_gate && lane == 0) shared_gate[t] = 1.0f / (1.0f + expf(-fresh(row + experts)));
     mx = ix_wave_max(mx);
+    const bool sigmoid = renormalize & IX_ROUTE_SIGMOID;  // (`renormalize` holds the selection mode's bits)
     float sum = 0.f;
 #pragma unroll
     for (int j = 0; j < SD_FEW_PER_LANE; ++j) {
       if (lane + 64 * j < experts) {
-        z[j] = expf(z[j] - mx);
+        z[j] = sigmoid ? 1.0f / (1.0f + expf(-z[j])) : expf(z[j] - mx);
         sum += z[j];
       }
     }
     sum = ix_wave_sum(sum);
-    const float inv_sum = 1.0f / sum;
+    const float inv_sum = sigmoid ? 1.0f : 1.0f / sum;
     if (groups_keep < n_groups) {  // (as in select_dispatch_body; lane g keeps the best score of group g)
       const int per = experts / n_groups;
       float best = -INFINITY;
+      const bool two = (renormalize & IX_ROUTE_GROUP_TOP2) && per > 1;  // (or the sum of its two largest)
       for (int gi = 0; gi < n_groups; ++gi) {
         float mg = -INFINITY;
+        int mi = 0x7fffffff;
 #pragma unroll
         for (int j = 0; j < SD_FEW_PER_LANE; ++j) {
           const int e = lane + 64 * j;
-          if (e < experts && e / per == gi) mg = fmaxf(mg, z[j]);
+          if (e < experts && e / per == gi && z[j] > mg) {
+            mg = z[j];
+            mi = e;
+          }
         }
-        mg = ix_wave_max(mg);
+        ix_wave_argmax(mg, mi);
+        if (two) {
+          float m2 = -INFINITY;
+#pragma unroll
+          for (int j = 0; j < SD_FEW_PER_LANE; ++j) {
+            const int e = lane + 64 * j;
+            if (e < experts && e / per == gi && e != mi) m2 = fmaxf(m2, z[j]);
+          }
+          mg += ix_wave_max(m2);
+        }
         if (lane == gi) best = mg;
       }
       bool kept = false;
@@ -335,7 +356,7 @@ select_dispatch_few(const float* logits, float* __restrict__ topk_w, int32_t* __
         chosen[t * k + slot] = bi;
       }
     }
-    const float f = ((renormalize && total > 0.f) ? 1.0f / total : 1.0f) * scale;
+    const float f = (((renormalize & IX_ROUTE_RENORMALIZE) && total > 0.f) ? 1.0f / total : 1.0f) * scale;
     if (lane < k) topk_w[t * k + lane] = mine_w * f;
   }
   __syncthreads();

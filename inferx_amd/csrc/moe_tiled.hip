@@ -54,7 +54,7 @@ __device__ __forceinline__ int tl_at(int row, int piece) { return row * TL_STRID
 template <bool GATE_UP, int NP, int NWW>
 __device__ __forceinline__ void
 tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ rows, int n_out, int width,
-           int e, int row0, int row_end, int tile, int col_block, __bf16* ws, __bf16* xs, int act) {
+           int e, int row0, int row_end, int tile, int col_block, __bf16* ws, __bf16* xs, int act, float glu_limit) {
   // (a and w are plain pointers on purpose: loads through `const __restrict__` ones may be moved by the
   // optimiser, which sinks them to their first use and so undoes the prefetch)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -249,7 +249,7 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float gate = acc[j][t][i];
-          v[i] = gate / (1.0f + __expf(-gate)) * acc[2 + j][t][i];
+          v[i] = ix_glu<true>(gate, acc[2 + j][t][i], glu_limit);
         }
         __bf16* dst = out + static_cast<int64_t>(r) * n_out + nb;
         if (nb + 4 <= n_out && vec) {
@@ -291,7 +291,7 @@ moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const in
                          const int32_t* __restrict__ rows,
                          const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
                          const int32_t* __restrict__ tile_info, int n_out, int width, int n_col_blocks,
-                         int act) {
+                         int act, float glu_limit) {
   __shared__ __attribute__((aligned(16))) __bf16 ws[2 * TL_WTILE(NWW)];
   __shared__ __attribute__((aligned(16))) __bf16 xs[2 * TL_XTILE(NWW)];
   // Workgroups go to the chip's eight dies in turn, by their number.  All column blocks of a row tile read the
@@ -305,23 +305,24 @@ moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const in
   const int held = min(TL_ROWS(NWW), row_end - row0);
   if (held <= 0) return;
   switch ((held + 31) >> 5) {  // pairs of sixteens of rows this tile holds
-    case 1: tiled_body<GATE_UP, 1, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
-    case 2: tiled_body<GATE_UP, 2, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
-    case 3: tiled_body<GATE_UP, 3, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
-    case 4: tiled_body<GATE_UP, 4, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
-    case 5: tiled_body<GATE_UP, 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
+    case 1: tiled_body<GATE_UP, 1, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act, glu_limit); break;
+    case 2: tiled_body<GATE_UP, 2, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act, glu_limit); break;
+    case 3: tiled_body<GATE_UP, 3, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act, glu_limit); break;
+    case 4: tiled_body<GATE_UP, 4, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act, glu_limit); break;
+    case 5: tiled_body<GATE_UP, 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act, glu_limit); break;
     default:  // (six pairs of sixteens in the wide form only)
-      tiled_body<GATE_UP, NWW == 4 ? 6 : 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act);
+      tiled_body<GATE_UP, NWW == 4 ? 6 : 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act, glu_limit);
       break;
   }
 }
 
 // The row-tile map must have been made for tiles of 160 rows, for the wide form of 192.  `wide`: see below.
 // gate_up: 0 a plain product, 1 gate|up rows with SwiGLU, 2 a plain product whose results pass the square of relu.
+// glu_limit > 0: the gate|up rows meet in the clamped form (`ix_glu`).
 extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, const int32_t* offsets,
                                     const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
                                     const int32_t* tile_info, int max_tiles, int64_t a_rows, int64_t n_out,
-                                    int64_t width, int gate_up, int wide, hipStream_t stream) {
+                                    int64_t width, int gate_up, int wide, float glu_limit, hipStream_t stream) {
   IX_REQUIRE(n_out > 0 && width > 0 && max_tiles >= 0, "sizes must be positive");
   IX_REQUIRE(width % 8 == 0, "the reduction width must be a multiple of 8 for the matrix-core kernel");
   IX_REQUIRE(n_out < (1 << 30) && width < (1 << 30), "sizes too large");
@@ -341,7 +342,7 @@ extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, con
 #define LAUNCH(GU, NWW)                                                                                             \
   hipLaunchKernelGGL((moe_grouped_tiled_kernel<GU, NWW>), grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w, \
                      (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width,         \
-                     n_col_blocks, gate_up == 2 ? 1 : 0)
+                     n_col_blocks, gate_up == 2 ? 1 : 0, glu_limit)
   if (nww == 4) {
     if (gate_up == 1) LAUNCH(true, 4);
     else LAUNCH(false, 4);

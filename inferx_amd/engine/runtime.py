@@ -94,7 +94,7 @@ class Runtime:
         return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < x.shape[0] <= self.SKINNY_ROWS
                 and x.shape[1] % 8 == 0 and x.is_contiguous() and w.is_contiguous())
 
-    def _skinny(self, x: torch.Tensor, w: torch.Tensor, gate_up: bool) -> torch.Tensor:
+    def _skinny(self, x: torch.Tensor, w: torch.Tensor, gate_up: bool, limit: float = 0.0) -> torch.Tensor:
         from .. import ops
         T = x.shape[0]
         plan = self._skinny_plans.get(T)
@@ -107,7 +107,7 @@ class Runtime:
         offsets, tile_map, tile_rows = plan
         n_out = w.shape[0] // 2 if gate_up else w.shape[0]
         out = self.empty((T, n_out))
-        ops.moe_grouped_mfma(x, w.unsqueeze(0), out, offsets, None, tile_map, tile_rows, gate_up, 4)
+        ops.moe_grouped_mfma(x, w.unsqueeze(0), out, offsets, None, tile_map, tile_rows, gate_up, 4, limit)
         return out
 
     def linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
@@ -126,14 +126,19 @@ class Runtime:
             return torch.matmul(x, w.t())
         return torch.matmul(x.to(torch.float32), w.to(torch.float32).t()).to(self.dtype)
 
-    def gated_linear(self, x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
-        """silu(x . Wg^T) * (x . Wu^T) for w_gate_up = [Wg; Wu] of shape [2 n, in] -> [T, n]."""
+    def gated_linear(self, x: torch.Tensor, w_gate_up: torch.Tensor, limit: float = 0.0,
+                     bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """silu(x . Wg^T) * (x . Wu^T) for w_gate_up = [Wg; Wu] of shape [2 n, in] -> [T, n].  `bias` (2 n numbers) is
+        added to both products first; with `limit` > 0 they meet in the clamped form instead (`ops.glu_bias`)."""
         from .. import ops
-        if self._skinny_ok(x, w_gate_up):
-            return self._skinny(x, w_gate_up, True)
+        if bias is None and self._skinny_ok(x, w_gate_up):
+            return self._skinny(x, w_gate_up, True, limit)
         gate_up = self.linear(x, w_gate_up)
         act = self.empty((x.shape[0], w_gate_up.shape[0] // 2))
-        ops.silu_mul(gate_up, act)
+        if bias is None and limit <= 0:
+            ops.silu_mul(gate_up, act)
+        else:
+            ops.glu_bias(gate_up, bias, act, limit)
         return act
 
     def linear_f32(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:

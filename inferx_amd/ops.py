@@ -314,10 +314,18 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 ROUTE_SMALL_TOKENS = 128
 
 
+def route_mode(renormalize: bool, sigmoid: bool = False, group_top2: bool = False) -> int:
+    """The bits that tell a router's selection what to do (IX_ROUTE_* of the kernels)."""
+    return (1 if renormalize else 0) | (2 if sigmoid else 0) | (4 if group_top2 else 0)
+
+
 def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor], topk_w: torch.Tensor,
               topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor], renormalize: bool, scale: float,
-              always: int = 0, groups: int = 1, groups_keep: int = 1) -> None:
+              always: int = 0, groups: int = 1, groups_keep: int = 1, sigmoid: bool = False,
+              group_top2: bool = False) -> None:
     """Router product, softmax and top-k in float32; optional sigmoid gate of the shared expert.
+    `sigmoid`: an expert's score is sigmoid(z) of its own logit instead of the softmax over all; `group_top2`: a
+    group's score is the sum of its two largest scores instead of its largest.
     `always`: that many further slots per token after the chosen ones (topk_w and topk_e are [T, k + always]), naming
     the experts E .. E + always - 1 with the shared gate's value (or 1) as their weight: experts that every token uses.
     `groups`, `groups_keep`: the experts form that many equal groups of neighbours, and only experts of the
@@ -345,7 +353,8 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
     _call("ix_moe_route", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
           _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(topk_w), _ptr(topk_e),
           _ptr(shared_gate if shared_gate_w is not None else None), _ptr(scratch), _i64(T), _i64(H), _i32(E), _i32(k),
-          _i32(1 if renormalize else 0), _f32(scale), _i32(always), _i32(groups), _i32(groups_keep), _stream())
+          _i32(route_mode(renormalize, sigmoid, group_top2)), _f32(scale), _i32(always), _i32(groups),
+          _i32(groups_keep), _stream())
 
 
 # the one-launch router: at most this many tokens, experts and bytes of one token as float32
@@ -375,7 +384,8 @@ def moe_route_dispatch(x: Optional[torch.Tensor], router_w: torch.Tensor, shared
                        topk_w: torch.Tensor, topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor],
                        renormalize: bool, scale: float, offsets: torch.Tensor, rows: torch.Tensor,
                        dest: torch.Tensor, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None,
-                       norm: Optional[tuple] = None, groups: int = 1, groups_keep: int = 1) -> None:
+                       norm: Optional[tuple] = None, groups: int = 1, groups_keep: int = 1, sigmoid: bool = False,
+                       group_top2: bool = False) -> None:
     """`moe_route` and `moe_dispatch` for up to 16 tokens in one launch: the router scores are spread over many
     workgroups, and the last one to finish its scores selects and groups (`route_one_launch_fits`).
 
@@ -417,7 +427,8 @@ def moe_route_dispatch(x: Optional[torch.Tensor], router_w: torch.Tensor, shared
               _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits),
               _ptr(_arrival_counter(x.device)), _i64(H), _ptr(topk_w), _ptr(topk_e),
               _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest),
-              _i32(T), _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(groups), _i32(groups_keep),
+              _i32(T), _i32(E), _i32(k), _i32(route_mode(renormalize, sigmoid, group_top2)), _f32(scale), _i32(groups),
+              _i32(groups_keep),
               _i32(tile_rows), _ptr(te), _ptr(tr), _ptr(ti), _stream())
     if norm is not None:
         _call("ix_moe_norm_route_dispatch_small", _ptr(h), _ptr(delta), _i32(_dt(x_out)), _ptr(gamma),
@@ -465,7 +476,7 @@ def moe_max_tiles(assignments: int, experts: int, tile_rows: int) -> int:
 
 def moe_grouped_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
                      rows: Optional[torch.Tensor], tile_map: torch.Tensor, tile_rows: int, gate_up: bool,
-                     k_split: int) -> None:
+                     k_split: int, glu_limit: float = 0.0) -> None:
     """Grouped product on the matrix cores (bfloat16), shapes as `moe_grouped_plain`; `tile_map` from `moe_dispatch`."""
     E = w.shape[0]
     A, n_out = out.shape
@@ -484,14 +495,16 @@ def moe_grouped_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
     _is_i32(tile_map, 2 * mt + 1)
     _call("ix_moe_grouped_mfma", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
           _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i32(tile_rows), _i64(n_out), _i64(K),
-          _i32(_epilogue(gate_up)), _i32(k_split), _stream())
+          _i32(_epilogue(gate_up)), _i32(k_split), _f32(glu_limit), _stream())
 
 
 def moe_grouped_dual(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
                      rows: Optional[torch.Tensor], tile_map: torch.Tensor, tile_rows: int, a_s: torch.Tensor,
-                     w_s: torch.Tensor, out_s: torch.Tensor, gate_up: bool) -> None:
+                     w_s: torch.Tensor, out_s: torch.Tensor, gate_up: bool, glu_limit: float = 0.0,
+                     glu_limit_s: float = 0.0) -> None:
     """`moe_grouped_mfma` (split reduction) for the routed experts and, in the same launch, the shared expert:
-    out_s = a_s . w_s^T (with SwiGLU when gate_up)."""
+    out_s = a_s . w_s^T (with SwiGLU when gate_up; `glu_limit`, `glu_limit_s`: the clamped form, for the routed
+    experts and for the shared one)."""
     E = w.shape[0]
     A, n_out = out.shape
     K = a.shape[1]
@@ -513,7 +526,8 @@ def moe_grouped_dual(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
     _is_i32(tile_map, 2 * mt + 1)
     _call("ix_moe_grouped_dual", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
           _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i32(tile_rows), _i64(n_out), _i64(K),
-          _ptr(a_s), _ptr(w_s), _ptr(out_s), _i32(T), _i64(n_out_s), _i64(K_s), _i32(1 if gate_up else 0), _stream())
+          _ptr(a_s), _ptr(w_s), _ptr(out_s), _i32(T), _i64(n_out_s), _i64(K_s), _i32(1 if gate_up else 0),
+          _f32(glu_limit), _f32(glu_limit_s), _stream())
 
 
 _no_library_kernel = set()  # shapes that the vendor's library has no kernel for
@@ -561,7 +575,8 @@ def moe_tiled_rows(wide: bool) -> int:
 
 
 def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
-                      rows: Optional[torch.Tensor], tile_map: torch.Tensor, gate_up: bool, wide: bool = False) -> None:
+                      rows: Optional[torch.Tensor], tile_map: torch.Tensor, gate_up: bool, wide: bool = False,
+                      glu_limit: float = 0.0) -> None:
     """Grouped product staged through LDS (bfloat16, many rows per expert); `tile_map` made for tiles of
     `moe_tiled_rows(wide)` rows.  `wide`: 256 instead of 128 weight rows per workgroup (the same sums in the same
     order; which rows share a tile, and with it where a row's sum starts, differs)."""
@@ -582,13 +597,15 @@ def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offse
     _is_i32(tile_map, 2 * mt + 1)
     _call("ix_moe_grouped_tiled", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
           _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i64(a.shape[0]), _i64(n_out), _i64(K),
-          _i32(_epilogue(gate_up)), _i32(1 if wide else 0), _stream())
+          _i32(_epilogue(gate_up)), _i32(1 if wide else 0), _f32(glu_limit), _stream())
 
 
 def moe_grouped_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
-                      rows: Optional[torch.Tensor], gate_up: bool) -> None:
+                      rows: Optional[torch.Tensor], gate_up: bool, glu_limit: float = 0.0) -> None:
     """Grouped product over device offsets.  gate_up: a [T, H] gathered through `rows`,
-    w [E, 2n, H], out [A, n] = silu(gate) * up.  Otherwise a [A, K], w [E, n, K], out [A, n]."""
+    w [E, 2n, H], out [A, n] = silu(gate) * up (with `glu_limit` > 0 the clamped form: gate = min(gate, limit),
+    up = clamp(up, -limit, limit), gate * sigmoid(1.702 gate) * (up + 1)).  Otherwise a [A, K], w [E, n, K],
+    out [A, n]."""
     E = w.shape[0]
     A, n_out = out.shape
     K = a.shape[1]
@@ -601,7 +618,7 @@ def moe_grouped_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offse
     else:
         _need(a.shape[0] >= A, "a has fewer rows than out")
     _call("ix_moe_grouped_plain", _ptr(a), _i32(_dt(a)), _ptr(w), _i32(_dt(w)), _ptr(out), _ptr(offsets), _ptr(rows),
-          _i64(A), _i32(E), _i64(n_out), _i64(K), _i32(_epilogue(gate_up)), _stream())
+          _i64(A), _i32(E), _i64(n_out), _i64(K), _i32(_epilogue(gate_up)), _f32(glu_limit), _stream())
 
 
 def moe_combine(y: torch.Tensor, dest: torch.Tensor, topk_w: torch.Tensor, shared: Optional[torch.Tensor],
@@ -1026,14 +1043,16 @@ def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ab: torch.Tens
 
 def head_norm_gate(x: torch.Tensor, out: torch.Tensor, eps: float, weight: Optional[torch.Tensor] = None,
                    gate: Optional[torch.Tensor] = None, x2: Optional[torch.Tensor] = None, lam: float = 0.0,
-                   mult: float = 1.0) -> None:
+                   mult: float = 1.0, weight_per_head: bool = False, gate_sigmoid: bool = False) -> None:
     """Per (token, head): o = x - lam * x2 (x2 optional); out = o / sqrt(mean(o^2) + eps) * weight * silu(gate) * mult.
-    x, x2 float32 [T, heads, vdim]; weight [vdim]; gate [T, >= heads * vdim] (rows may be strided) and out
+    x, x2 float32 [T, heads, vdim]; weight [vdim] (`weight_per_head`: [heads, vdim]); `gate_sigmoid`: sigmoid(gate)
+    instead of silu(gate); gate [T, >= heads * vdim] (rows may be strided) and out
     [T, heads * vdim] of the run's type."""
     T, heads, vdim = x.shape
     _need(x.dtype == torch.float32 and (x2 is None or (x2.dtype == torch.float32 and x2.shape == x.shape)), "x, x2 float32")
     _need(out.shape == (T, heads * vdim), "out must be [T, heads * vdim]")
-    _need(weight is None or weight.numel() == vdim, "one weight per value column")
+    _need(weight is None or weight.numel() == (heads * vdim if weight_per_head else vdim),
+          "one weight per value column (of every head, with weight_per_head)")
     stride = 0
     if gate is not None:
         _need(gate.dim() == 2 and gate.shape == (T, heads * vdim) and gate.stride(1) == 1 and gate.dtype == out.dtype
@@ -1041,7 +1060,7 @@ def head_norm_gate(x: torch.Tensor, out: torch.Tensor, eps: float, weight: Optio
         stride = gate.stride(0)
     _call("ix_head_norm_gate", _ptr(x), _ptr(x2), _f32(lam), _ptr(weight), _i32(_dt(weight) if weight is not None else F32),
           gate.data_ptr() if gate is not None else None, _i64(stride), _ptr(out), _i32(_dt(out)), _i64(T), _i32(heads),
-          _i32(vdim), _f32(eps), _f32(mult), _stream())
+          _i32(vdim), _f32(eps), _f32(mult), _i32(1 if weight_per_head else 0), _i32(1 if gate_sigmoid else 0), _stream())
 
 
 def attention_diff_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -1103,3 +1122,137 @@ def attention_diff_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
           _i64(T), _i32(n_tiles), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(vd), _i32(page_size),
           _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(keep_first), _f32(lam), _f32(eps), _f32(mult),
           _i32(1 if grouped else 0), _stream())
+
+
+# ---- a gated product's activation with biases and limits; two branches added to the stream ---------------------
+def glu_bias(gate_up: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, limit: float = 0.0) -> None:
+    """out[t, i] = glu(gate_up[t, i] + bias[i], gate_up[t, W + i] + bias[W + i]); glu(g, u) = silu(g) * u, or with
+    `limit` > 0 the clamped form g' sigmoid(1.702 g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit)."""
+    T, W2 = gate_up.shape
+    _need(W2 % 2 == 0 and out.shape == (T, W2 // 2) and out.dtype == gate_up.dtype, "shape or dtype mismatch")
+    _need(bias is None or bias.numel() == W2, "the bias holds the gate's numbers, then the up's")
+    _call("ix_glu_bias", _ptr(gate_up), _ptr(bias), _i32(_dt(bias) if bias is not None else F32), _ptr(out),
+          _i32(_dt(out)), _i64(T), _i64(W2 // 2), _f32(limit), _stream())
+
+
+def add_branches(h: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None,
+                 bias: Optional[torch.Tensor] = None) -> None:
+    """h [T, W] float32 += a + b + bias (b and bias optional), summed in float32."""
+    _need(h.dtype == torch.float32 and h.dim() == 2, "the residual stream is float32 [T, W]")
+    _need(a.shape == h.shape and (b is None or (b.shape == h.shape and b.dtype == a.dtype)), "the branches have h's shape")
+    _need(bias is None or bias.numel() == h.shape[1], "one bias per column")
+    _call("ix_add_branches", _ptr(h), _ptr(a), _ptr(b), _i32(_dt(a)), _ptr(bias),
+          _i32(_dt(bias) if bias is not None else F32), _i64(h.shape[0]), _i64(h.shape[1]), _stream())
+
+
+# ---- recurrent mixers with a matrix of state per head ---------------------------------------------------------------
+def linear_state(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, rows: StepRows,
+                 out: torch.Tensor, heads: int, dim: int, vdim: int, w_rows: Optional[torch.Tensor] = None,
+                 w_head: Optional[torch.Tensor] = None, a_rows: Optional[torch.Tensor] = None,
+                 b_rows: Optional[torch.Tensor] = None, silu: bool = False) -> None:
+    """S <- diag(w) S - a (b^T S) + k v^T;  o = S^T r, over the rows of a step, request by request, from and to
+    `state` (a float32 view [slots, >= heads * vdim * dim], a head's matrix kept [vdim][dim]).  r, k [T, heads * dim],
+    v [T, heads * vdim] of the run's type (rows may be strided), through silu first if `silu`.  The decay w comes per
+    row and key channel (`w_rows` float32 [T, heads * dim]) or per head (`w_head` float32 [heads]); the correction's
+    vectors `a_rows`, `b_rows` (float32 [T, heads * dim]) come together or not at all.  out float32 [T, heads, vdim]."""
+    T = r.shape[0]
+    for t, n in ((r, heads * dim), (k, heads * dim), (v, heads * vdim)):
+        _need(t.dim() == 2 and t.shape == (T, n) and t.stride(1) == 1 and t.dtype == r.dtype and t.is_cuda, "r, k or v shape")
+    for t in (w_rows, a_rows, b_rows):
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (T, heads * dim) and t.is_contiguous()),
+              "the rows of decays and corrections must be float32 [T, heads * dim]")
+    _need((w_rows is None) != (w_head is None), "the decay comes per row and channel or per head")
+    _need(w_head is None or (w_head.dtype == torch.float32 and w_head.numel() == heads), "w_head must be float32 [heads]")
+    _need((a_rows is None) == (b_rows is None), "the correction's two vectors come together")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= heads * dim * vdim, "the state must be float32 [slots, >= heads * dim * vdim]")
+    _need(out.dtype == torch.float32 and out.shape == (T, heads, vdim) and out.is_contiguous(), "out must be float32 [T, heads, vdim]")
+    rows.check(T)
+    S = rows.q_start.numel() - 1
+    _call("ix_linear_state", r.data_ptr(), k.data_ptr(), v.data_ptr(), _i32(_dt(r)), _i64(r.stride(0)), _i64(k.stride(0)),
+          _i64(v.stride(0)), _ptr(w_rows), _ptr(w_head), _ptr(a_rows), _ptr(b_rows), state.data_ptr(),
+          _i64(state.stride(0)), _ptr(rows.q_start), _ptr(rows.state_slots), _ptr(out), _i64(T), _i32(S), _i32(heads),
+          _i32(dim), _i32(vdim), _i32(1 if silu else 0), _stream())
+
+
+def delta_operands(w_logit: torch.Tensor, w_bias: torch.Tensor, a_logit: torch.Tensor, a_bias: torch.Tensor,
+                   k: torch.Tensor, w: torch.Tensor, a: torch.Tensor, u: torch.Tensor, heads: int, dim: int,
+                   decay_scale: float, unit_eps: float) -> None:
+    """Per token, head and key channel, float32 [T, heads * dim]: w = exp(-decay_scale sigmoid(w_logit + w_bias)),
+    u = k / sqrt(sum over the head of k^2 + unit_eps), a = sigmoid(a_logit + a_bias) u.  w_logit float32; a_logit and
+    k of the run's type (rows may be strided)."""
+    T, C = w_logit.shape
+    _need(C == heads * dim and w_logit.dtype == torch.float32 and w_logit.is_contiguous(), "w_logit must be float32 [T, heads * dim]")
+    for t in (a_logit, k):
+        _need(t.dim() == 2 and t.shape == (T, C) and t.stride(1) == 1 and t.dtype == k.dtype and t.is_cuda, "a_logit or k shape")
+    _need(w_bias.numel() == C and a_bias.numel() == C, "one bias per channel")
+    for t in (w, a, u):
+        _need(t.dtype == torch.float32 and t.shape == (T, C) and t.is_contiguous(), "results are float32 [T, heads * dim]")
+    _call("ix_delta_operands", _ptr(w_logit), _ptr(w_bias), _i32(_dt(w_bias)), a_logit.data_ptr(), _i64(a_logit.stride(0)),
+          _ptr(a_bias), _i32(_dt(a_bias)), k.data_ptr(), _i64(k.stride(0)), _i32(_dt(k)), _ptr(w), _ptr(a), _ptr(u),
+          _i64(T), _i32(heads), _i32(dim), _f32(decay_scale), _f32(unit_eps), _stream())
+
+
+def tanh_(x: torch.Tensor) -> None:
+    """x = tanh(x) in place, float32."""
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "x must be float32")
+    _call("ix_tanh_inplace", _ptr(x), _i64(x.numel()), _stream())
+
+
+# ---- attention over a compressed cache ------------------------------------------------------------------------------
+def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, norm_w: torch.Tensor, eps: float,
+                   cos_sin: Optional[torch.Tensor], slots: Optional[torch.Tensor], cache: torch.Tensor, heads: int,
+                   rot_dim: int, rank: int) -> None:
+    """Per token: the last `rot_dim` numbers of every head of q [T, heads * q_dim] are rotated in place (pairs
+    (2i, 2i + 1), i < cos_sin.shape[1]; float32 table [T, pairs, 2]); the first `rank` numbers of the dkv row pass an
+    RMS norm with `norm_w` (float32 sums), its last rot_dim are rotated likewise, and [c | kr] goes to row slots[t] of
+    `cache` [pages, 1, page_size, rank + rot_dim]."""
+    T = q.shape[0]
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.is_cuda and q.shape[1] % heads == 0, "q must be rows of heads * q_dim")
+    q_dim = q.shape[1] // heads
+    _need(dkv.dim() == 2 and dkv.shape[0] == T and dkv.shape[1] >= rank + rot_dim and dkv.stride(1) == 1
+          and dkv.dtype == q.dtype and dkv.is_cuda, "dkv must be rows of at least rank + rot_dim numbers of q's type")
+    _need(norm_w.numel() == rank, "one norm weight per latent number")
+    pairs = 0
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[0] == T and cos_sin.shape[2] == 2
+              and cos_sin.is_contiguous(), "the rotation table must be float32 [T, pairs, 2]")
+        pairs = cos_sin.shape[1]
+    _need(2 * pairs <= rot_dim <= q_dim, "the rotated pairs must fit into the rotated part")
+    _need(cache.dtype == q.dtype and cache.dim() == 4 and cache.shape[1] == 1 and cache.shape[3] == rank + rot_dim
+          and cache.is_contiguous(), "the cache must be [pages, 1, page_size, rank + rot_dim] of q's type")
+    if slots is not None:
+        _is_i32(slots, T)
+    _call("ix_latent_prepare", q.data_ptr(), _i64(q.stride(0)), dkv.data_ptr(), _i64(dkv.stride(0)), _i32(_dt(q)), _ptr(norm_w),
+          _i32(_dt(norm_w)), _f32(eps), _ptr(cos_sin), _i32(pairs), _ptr(slots), _ptr(cache), _i64(T), _i32(heads),
+          _i32(q_dim), _i32(rot_dim), _i32(rank), _stream())
+
+
+def _head_rows(t: torch.Tensor, tokens: int, heads: int, n: int, what: str):
+    """(token stride, head stride) of a tensor indexed [token, head, i] whose last dimension is dense."""
+    _need(t.dim() == 3 and t.shape[0] == tokens and t.shape[1] == heads and t.shape[2] >= n and t.stride(2) == 1
+          and t.is_cuda, f"{what} must be indexed [token, head, i] with a dense last dimension")
+    return t.stride(0), t.stride(1)
+
+
+def latent_attention_plain(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
+                           seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, rank: int,
+                           rot_dim: int, scale: float) -> None:
+    """Causal attention of queries [token, head] over cached rows [c | kr]: score = (q_lat . c + q_rot . kr) * scale,
+    softmax in float32, out = sum of weights * c.  q_lat, out [token, head, rank] and q_rot [token, head, rot_dim] are
+    views with any token and head strides; cache [pages, 1, page_size, rank + rot_dim]."""
+    T, heads = q_lat.shape[0], q_lat.shape[1]
+    ql_t, ql_h = _head_rows(q_lat, T, heads, rank, "q_lat")
+    qr_t, qr_h = _head_rows(q_rot, T, heads, rot_dim, "q_rot")
+    o_t, o_h = _head_rows(out, T, heads, rank, "out")
+    _need(q_rot.dtype == q_lat.dtype and out.dtype == q_lat.dtype and cache.dtype == q_lat.dtype, "one element type")
+    _need(cache.dim() == 4 and cache.shape[1] == 1 and cache.shape[3] == rank + rot_dim and cache.is_contiguous(),
+          "the cache must be [pages, 1, page_size, rank + rot_dim]")
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    _is_i32(block_table)
+    _is_i32(seq_of_token, T)
+    _is_i32(positions, T)
+    _call("ix_latent_attention_plain", q_lat.data_ptr(), _i64(ql_t), _i64(ql_h), q_rot.data_ptr(), _i64(qr_t), _i64(qr_h),
+          _ptr(cache), _i32(_dt(q_lat)), _ptr(block_table), _ptr(seq_of_token), _ptr(positions), out.data_ptr(),
+          _i64(o_t), _i64(o_h), _i64(T), _i32(heads), _i32(rank), _i32(rot_dim), _i32(cache.shape[2]),
+          _i32(block_table.shape[1]), _f32(scale), _stream())

@@ -9,7 +9,11 @@ says so gets norm2 unapplied (`LazyNorm`) and applies it in its first kernel.
 """
 from __future__ import annotations
 
-from .base import Block, LazyNorm, register_part, resolve_delta
+import torch
+
+from .. import ops
+from .base import Block, LazyDelta, LazyNorm, register_part, resolve_delta
+from .dense_mlp import BiasedDelta
 from .norm import NormedDelta
 
 
@@ -100,6 +104,63 @@ class SandwichNormBlock(Block):
         return NormedDelta(self.feed_forward.forward(ctx, x), self.feed_forward_post_norm)
 
 
+class BranchSum(LazyDelta):
+    """The sum of two branches' results, not formed yet: `first` a tensor, `second` a tensor, a `BiasedDelta` or any
+    other sum that is not formed (the experts').  Whoever adds it to the stream adds the parts one by one, in
+    float32: the first (with a tensor second, and its bias, in the same pass), then what the second knows to fuse
+    with the norm that follows."""
+
+    def __init__(self, first, second):
+        self.first, self.second = first, second
+
+    def _add_first(self, ctx, h):
+        """h += first (+ second where that is a tensor, with its bias); returns what is still to be added."""
+        second = self.second
+        if isinstance(second, BiasedDelta):
+            ops.add_branches(h, self.first, second.tensor, second.bias)
+            return None
+        if isinstance(second, LazyDelta):
+            ops.add_branches(h, self.first)
+            return second
+        ops.add_branches(h, self.first, second)
+        return None
+
+    def materialize(self, ctx):
+        total = torch.zeros(tuple(self.first.shape), dtype=torch.float32, device=self.first.device)
+        rest = self._add_first(ctx, total)
+        if rest is not None:
+            ops.add_branches(total, rest.materialize(ctx))
+        return total
+
+    def add_rmsnorm(self, ctx, h, weight, eps, rows, out) -> bool:
+        """The stream takes the whole sum here, also where only picked rows are normalised (the model's last norm:
+        nobody reads the stream after it)."""
+        rest = self._add_first(ctx, h)
+        if rest is None or not rest.add_rmsnorm(ctx, h, weight, eps, rows, out):
+            ops.add_rmsnorm(h, None if rest is None else rest.materialize(ctx), weight, out, eps, rows)
+        return True
+
+
+class ParallelBlock(Block):
+    """One norm, and both branches read its result:
+
+        x = norm(h + pending);   pending = mixer(x) + feed_forward(x)
+
+    The feed-forward may be left out.  The sum travels unformed (`BranchSum`) to the next norm."""
+
+    graph_safe = True
+    part_kinds = {"norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+    optional_parts = ("feed_forward",)
+
+    def forward(self, ctx, h, pending, caches):
+        x = self.norm.forward(ctx, h, pending)
+        a = self.mixer.forward(ctx, x, caches.get("mixer"))
+        if self.feed_forward is None:
+            return a
+        return BranchSum(resolve_delta(ctx, a), self.feed_forward.forward(ctx, x))
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)
 register_part("block", "sandwich_norm", SandwichNormBlock)
 register_part("block", "prenorm_gained", GainedPreNormBlock)

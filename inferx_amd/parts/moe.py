@@ -11,6 +11,10 @@ float32 from the product on.
 Two options beside that: experts without a gate (`gated=False`: down(act(up x)) with act the square of relu, weights
 w13 [E, mi, H]) and a router that chooses among groups (`groups`, `groups_keep`: the experts form equal groups of
 neighbours, a group's score is its best expert's, and only experts of the best `groups_keep` groups can be chosen).
+Further: `score` "sigmoid" (an expert's score is the sigmoid of its own logit, not the softmax over all),
+`group_score` "top2" (a group's score is the sum of its two best experts'), and the activation "clamped_glu" with
+`limit` (and `shared_limit` for the shared expert): g = min(gate, limit), u = clamp(up, -limit, limit),
+g sigmoid(1.702 g) (u + 1).
 """
 from __future__ import annotations
 
@@ -53,7 +57,8 @@ class MoeFeedForward(FeedForward):
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_width: int, shared_width: int = 0,
                  shared_gated: bool = True, renormalize: bool = False, routed_scale: float = 1.0,
                  init_std: float = 0.02, gated: bool = True, activation: Optional[str] = None, groups: int = 1,
-                 groups_keep: int = 1):
+                 groups_keep: int = 1, score: str = "softmax", group_score: str = "best", limit: float = 0.0,
+                 shared_limit: Optional[float] = None):
         if not 0 < top_k <= num_experts:
             raise ValueError(f"top_k {top_k} must be between 1 and num_experts {num_experts}")
         if num_experts > 1024 or top_k > 32:
@@ -64,9 +69,17 @@ class MoeFeedForward(FeedForward):
         self.routed_scale, self.init_std = float(routed_scale), float(init_std)
         self.gated = bool(gated)
         activation = activation or ("silu" if self.gated else "relu2")
-        if (self.gated, activation) not in ((True, "silu"), (False, "relu2")):
+        if (self.gated, activation) not in ((True, "silu"), (True, "clamped_glu"), (False, "relu2")):
             raise ValueError(f"experts {'with' if self.gated else 'without'} a gate and the activation {activation!r}: "
-                             "a gate goes with silu, no gate with relu2 (the square of relu)")
+                             "a gate goes with silu or clamped_glu, no gate with relu2 (the square of relu)")
+        if score not in ("softmax", "sigmoid") or group_score not in ("best", "top2"):
+            raise ValueError(f"router scores {score!r} (softmax or sigmoid), group scores {group_score!r} (best or top2)")
+        self.sigmoid_scores, self.group_top2 = score == "sigmoid", group_score == "top2"
+        # the clamped activation's limits (0: the activation is silu(gate) * up)
+        self.limit = float(limit) if activation == "clamped_glu" else 0.0
+        self.shared_limit = self.limit if shared_limit is None or activation != "clamped_glu" else float(shared_limit)
+        if activation == "clamped_glu" and (self.limit <= 0 or self.shared_limit <= 0):
+            raise ValueError("the clamped activation needs a positive limit")
         if not self.gated and shared_width:
             raise ValueError("a shared expert needs gated experts")
         self.activation = activation
@@ -81,7 +94,7 @@ class MoeFeedForward(FeedForward):
         # pieces of the routed experts' width that the shared expert is cut into for steps of middling size, or 0
         self.shared_pieces = self.shared_width // self.expert_width if (
             self.shared_width > 0 and self.shared_width % self.expert_width == 0
-            and self.shared_width // self.expert_width <= 32) else 0
+            and self.shared_width // self.expert_width <= 32 and self.shared_limit == self.limit) else 0
         self.w13_all = self.w2_all = None  # routed experts, then the shared expert's pieces
         self.w_router = self.w13 = self.w2 = None
         self.w_shared_gate_up = self.w_shared_down = self.w_shared_gate = None
@@ -140,7 +153,7 @@ class MoeFeedForward(FeedForward):
         topk_e = rt.empty((T, k), torch.int32)
         gate = rt.empty((T,), torch.float32) if self.w_shared_gate is not None else None
         ops.moe_route(x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate, self.renormalize, self.routed_scale,
-                      always, self.groups, self.groups_keep)
+                      always, self.groups, self.groups_keep, self.sigmoid_scores, self.group_top2)
         return topk_w, topk_e, gate
 
     def _tile_rows(self, ctx, x) -> int:
@@ -173,14 +186,14 @@ class MoeFeedForward(FeedForward):
         act = rt.empty((A, self.expert_width))
         y = rt.empty((A, self.hidden_size))
         if tile_rows == ops.moe_tiled_rows(self.wide_tiles):  # many rows per expert: operands staged through LDS
-            ops.moe_grouped_tiled(x, w13, act, offsets, rows, tile_map, self.first_epilogue, self.wide_tiles)
+            ops.moe_grouped_tiled(x, w13, act, offsets, rows, tile_map, self.first_epilogue, self.wide_tiles, self.limit)
             ops.moe_grouped_tiled(act, w2, y, offsets, None, tile_map, False, self.wide_tiles)
         elif tile_rows:
             # few rows: the weights are the traffic, the reduction is split over a workgroup's four wavefronts
-            ops.moe_grouped_mfma(x, w13, act, offsets, rows, tile_map, tile_rows, self.first_epilogue, 4)
+            ops.moe_grouped_mfma(x, w13, act, offsets, rows, tile_map, tile_rows, self.first_epilogue, 4, self.limit)
             ops.moe_grouped_mfma(act, w2, y, offsets, None, tile_map, tile_rows, False, 4)
         else:
-            ops.moe_grouped_plain(x, w13, act, offsets, rows, gate_up=self.first_epilogue)
+            ops.moe_grouped_plain(x, w13, act, offsets, rows, gate_up=self.first_epilogue, glu_limit=self.limit)
             ops.moe_grouped_plain(act, w2, y, offsets, None, gate_up=False)
         return y
 
@@ -193,14 +206,15 @@ class MoeFeedForward(FeedForward):
     def experts_and_shared(self, ctx, x, offsets, rows, tile_map, tile_rows):
         rt, A, T = ctx.rt, rows.numel(), x.shape[0]
         act, sact = rt.empty((A, self.expert_width)), rt.empty((T, self.shared_width))
-        ops.moe_grouped_dual(x, self.w13, act, offsets, rows, tile_map, tile_rows, x, self.w_shared_gate_up, sact, True)
+        ops.moe_grouped_dual(x, self.w13, act, offsets, rows, tile_map, tile_rows, x, self.w_shared_gate_up, sact, True,
+                             self.limit, self.shared_limit)
         y, sout = rt.empty((A, self.hidden_size)), rt.empty((T, self.hidden_size))
         ops.moe_grouped_dual(act, self.w2, y, offsets, None, tile_map, tile_rows, sact, self.w_shared_down, sout, False)
         return y, sout
 
     def shared(self, ctx, x):
         rt = ctx.rt
-        return rt.linear(rt.gated_linear(x, self.w_shared_gate_up), self.w_shared_down)
+        return rt.linear(rt.gated_linear(x, self.w_shared_gate_up, limit=self.shared_limit), self.w_shared_down)
 
     def route_and_dispatch(self, ctx, x, tile_rows: int, norm=None, always: int = 0):
         """`route` then `dispatch`; for the few tokens of a decoding step in one launch, and the norm before the
@@ -220,7 +234,7 @@ class MoeFeedForward(FeedForward):
         tile_map = rt.empty((2 * ops.moe_max_tiles(T * k, E, tile_rows) + 1,), torch.int32) if tile_rows else None
         ops.moe_route_dispatch(None if norm else x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate,
                                self.renormalize, self.routed_scale, offsets, rows, dest, tile_rows, tile_map, norm,
-                               self.groups, self.groups_keep)
+                               self.groups, self.groups_keep, self.sigmoid_scores, self.group_top2)
         return topk_w, topk_e, gate, offsets, rows, dest, tile_map
 
     def _routes_in_one_launch(self, tokens: int) -> bool:

@@ -16,15 +16,18 @@ from .base import LazyDelta, Norm, ParamSpec, register_part
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, width: int, eps: float):
-        self.width, self.eps = int(width), float(eps)
+    def __init__(self, width: int, eps: float, scalar: bool = False):
+        """`scalar`: the weight is ONE number for all coordinates (a tensor without dimensions), spread over the
+        width when it is bound, so that every kernel that applies an RMS norm takes it as it is."""
+        self.width, self.eps, self.scalar = int(width), float(eps), bool(scalar)
         self.weight = None
 
     def param_specs(self) -> List[ParamSpec]:
-        return [ParamSpec("weight", (self.width,), init="ones")]
+        return [ParamSpec("weight", () if self.scalar else (self.width,), init="ones")]
 
     def bind(self, tensors, rt) -> None:
-        self.weight = tensors["weight"].contiguous()
+        w = tensors["weight"]
+        self.weight = w.reshape(1).expand(self.width).contiguous() if self.scalar else w.contiguous()
 
     def rms_operands(self):
         return self.weight, self.eps
