@@ -18,6 +18,18 @@ import torch
 F = torch.float64
 
 
+def exact(x):
+    return x
+
+
+def bfloat16(x):
+    """x rounded to bfloat16 (nearest even) and back: what keeping an activation in 16 bits does to it."""
+    return x.to(torch.bfloat16).to(F)
+
+
+_S = exact  # what keeping an activation between two operations does to it (`forward(store=...)` sets it)
+
+
 def rms_unit(x, eps):
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
 
@@ -43,28 +55,30 @@ def rotate_pairs(x, positions, dims, base):
 def latent_attention(x, w, m, eps, positions):
     T = x.shape[0]
     H, d, r, vd, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
-    q = (x @ w["q"].T).view(T, H, d + r)
-    dkv = x @ w["dkv"].T
-    c = rms_unit(dkv[:, :rank], eps) * w["dkv.norm"]
-    rot = m["rot"]
-    kr = rotate_pairs(dkv[:, rank:], positions, rot["dims"], rot["base"])
-    q_rot = rotate_pairs(q[:, :, d:], positions, rot["dims"], rot["base"])
-    k = (c @ w["uk"].T).view(T, H, d)
-    v = (c @ w["uv"].T).view(T, H, vd)
+    q = _S(x @ w["q"].T).view(T, H, d + r)
+    dkv = _S(x @ w["dkv"].T)
+    c = _S(rms_unit(dkv[:, :rank], eps) * w["dkv.norm"])
+    rot = m.get("rot")
+    kr, q_rot = dkv[:, rank:], q[:, :, d:]
+    if rot is not None:
+        kr = _S(rotate_pairs(kr, positions, rot["dims"], rot["base"]))
+        q_rot = _S(rotate_pairs(q_rot, positions, rot["dims"], rot["base"]))
+    k = _S(c @ w["uk"].T).view(T, H, d)
+    v = _S(c @ w["uv"].T).view(T, H, vd)
     score = (torch.einsum("ihd,jhd->hij", q[:, :, :d], k) + torch.einsum("ihr,jr->hij", q_rot, kr)) * m["scale"]
     seen = positions[None, :] <= positions[:, None]
     score = score.masked_fill(~seen[None], -math.inf)
     p = torch.softmax(score, -1)
-    o = torch.einsum("hij,jhv->ihv", p, v).reshape(T, H * vd)
-    return o @ w["o"].T
+    o = _S(torch.einsum("hij,jhv->ihv", p, v).reshape(T, H * vd))
+    return _S(o @ w["o"].T)
 
 
 def general_delta(x, w, m, eps):
     T = x.shape[0]
     H, d = m["heads"], m["dim"]
-    r, k, v = [(x @ w[n].T).view(T, H, d) for n in ("r", "k", "v")]
+    r, k, v = [_S(x @ w[n].T).view(T, H, d) for n in ("r", "k", "v")]
     decay = torch.exp(-math.exp(-0.5) * torch.sigmoid(torch.tanh(x @ w["w1"].T) @ w["w2"].T + w["w0"])).view(T, H, d)
-    a = torch.sigmoid(x @ w["a"].T + w["a.b"]).view(T, H, d)
+    a = torch.sigmoid(_S(x @ w["a"].T) + w["a.b"]).view(T, H, d)
     u = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
     S = torch.zeros(H, d, d, dtype=F)
     o = torch.zeros(T, H, d, dtype=F)
@@ -73,30 +87,30 @@ def general_delta(x, w, m, eps):
         read = torch.einsum("hi,hij->hj", u[t], old)
         S = decay[t][:, :, None] * old - (a[t] * u[t])[:, :, None] * read[:, None, :] + k[t][:, :, None] * v[t][:, None, :]
         o[t] = torch.einsum("hij,hi->hj", S, r[t])
-    y = rms_unit(o, eps).reshape(T, H * d) * w["norm"] * torch.sigmoid(x @ w["g"].T)
-    return y @ w["o"].T
+    y = _S(rms_unit(o, eps).reshape(T, H * d) * w["norm"] * torch.sigmoid(_S(x @ w["g"].T)))
+    return _S(y @ w["o"].T)
 
 
 def lightning(x, w, m, eps):
     T = x.shape[0]
     H, d, vd = m["heads"], m["dim"], m["vdim"]
     silu = torch.nn.functional.silu
-    q, k = silu(x @ w["q"].T).view(T, H, d), silu(x @ w["k"].T).view(T, H, d)
-    v = silu(x @ w["v"].T).view(T, H, vd)
+    q, k = silu(_S(x @ w["q"].T)).view(T, H, d), silu(_S(x @ w["k"].T)).view(T, H, d)
+    v = silu(_S(x @ w["v"].T)).view(T, H, vd)
     decay = torch.tensor(m["decay"], dtype=F)
     S = torch.zeros(H, d, vd, dtype=F)
     o = torch.zeros(T, H, vd, dtype=F)
     for t in range(T):
         S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
         o[t] = torch.einsum("hij,hi->hj", S, q[t])
-    y = rms_unit(o.reshape(T, H * vd), eps) * w["norm"] * torch.sigmoid(x @ w["g"].T)
-    return y @ w["o"].T
+    y = _S(rms_unit(o.reshape(T, H * vd), eps) * w["norm"] * torch.sigmoid(_S(x @ w["g"].T)))
+    return _S(y @ w["o"].T)
 
 
 def clamped_glu(x, gate, up, down, limit, gate_b=0.0, up_b=0.0, down_b=0.0):
     g = torch.clamp(x @ gate.T + gate_b, max=limit)
     u = torch.clamp(x @ up.T + up_b, -limit, limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ down.T + down_b
+    return _S(_S(g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ down.T + down_b)
 
 
 def dense_ff(x, w, f):
@@ -147,19 +161,29 @@ def sub(tensors, prefix):
     return {k[len(prefix):]: v.to(F) for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(config, tensors, tokens, chosen=None, keep_layers=False, keep_router=None):
+def forward(config, tensors, tokens, chosen=None, keep_layers=False, keep_router=None, store=exact):
     """Logits [T, vocab] of one sequence from position 0; with `keep_layers` also the stream after every layer run.
     `chosen`: {layer run: experts [T, top]} from outside; `keep_router`: a dict that receives every routed layer
-    run's scores [T, E]."""
+    run's scores [T, E].  `store=bfloat16`: a model of a 16-bit run, in which every activation kept between two
+    operations is rounded (the stream, the norms' sums, scores, routers and recurrences stay as they are)."""
+    global _S
+    _S = store
+    try:
+        return _forward(config, tensors, tokens, chosen, keep_layers, keep_router)
+    finally:
+        _S = exact
+
+
+def _forward(config, tensors, tokens, chosen, keep_layers, keep_router):
     eps = config["norm"]["eps"]
     ids = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(len(ids))
-    h = tensors["embed"].to(F)[ids] * config["embedding"]["scale"]
+    h = tensors["embed"].to(F)[ids] * config.get("embedding", {}).get("scale", 1.0)
     after = []
     for i, layer in enumerate(config["layers"]):
         src = layer.get("weights_of", i)
         p = f"l{src}."
-        x = scalar_norm(h, tensors[p + "norm1"].to(F), eps)
+        x = _S(scalar_norm(h, tensors[p + "norm1"].to(F), eps))
         delta = MIXERS[layer["type"]](x, sub(tensors, p + "mix."), layer["mixer"], eps, positions)
         f = layer.get("mlp")
         if f is not None:
@@ -172,5 +196,5 @@ def forward(config, tensors, tokens, chosen=None, keep_layers=False, keep_router
                 delta = delta + moe_ff(x, w, f, None if chosen is None else chosen.get(i))
         h = h + delta
         after.append(h.clone())
-    logits = scalar_norm(h, tensors["final.norm"].to(F), eps) @ tensors["head"].to(F).T
+    logits = _S(scalar_norm(h, tensors["final.norm"].to(F), eps)) @ tensors["head"].to(F).T
     return (logits, torch.stack(after)) if keep_layers else logits
