@@ -176,3 +176,270 @@ extern "C" int ix_latent_attention_plain(const void* ql, int64_t ql_t, int64_t q
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_latent_attention_plain");
 }
+
+// ---------------------------------------------------------------------------
+// The same attention on the matrix cores (bfloat16; rank + rot_dim a multiple of 32 up to 576, rank a multiple of
+// 16 up to 512).  All heads read the same cached rows, so a workgroup of four wavefronts shares them through LDS:
+// 32 keys a round, the row [c | kr] as it is for the scores and the latent part once more transposed ([d][key])
+// for the weighted sum, so that both products take their operands in 16-byte pieces:
+//
+//     S^T[key][column] = K[key][:] . Q[column][:]             (A = key rows, B = the column's query, in registers)
+//     O^T[d][column]  += C^T[d][key] P^T[key][column]          (A = transposed latent rows, B = the weights)
+//
+// v_mfma_f32_16x16x32_bf16 leaves lane l with column l % 16 and rows 4 (l / 16) + i.  Row m of the first 16 keys
+// of a round is key 8 (m / 4) + m % 4, of the second key 8 (m / 4) + 4 + m % 4, so a lane holds the scores of keys
+// 8 (l / 16) .. + 7 of its column: the B operand of the second product as it stands.  Softmax online, float32, per
+// column; a lane's accumulators all belong to its column, so rescaling is a multiplication by the lane's factor.
+//
+// What a column is: prompt portions (DEC false): a workgroup takes 16 consecutive rows of the step and four heads,
+// a wavefront one head, a column one row.  Rows of several requests in a tile are worked request by request (the
+// other rows' keys all masked: they change nothing).  One token per request (DEC true): a workgroup takes one token
+// and one slice of its keys, a wavefront sixteen heads, a column one head; slices leave (max, sum, unnormalised
+// sums) for `attn_combine_kernel`.  The next round's rows are on their way from memory while a round is multiplied.
+typedef __bf16 lat_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 lat_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float lat_f32x4 __attribute__((ext_vector_type(4)));
+
+#define LATM_KEYS 32
+#define LATM_KPAD 8      // numbers between key rows in LDS (keeps 16-byte pieces aligned, spreads the banks)
+#define LATM_VSTRIDE 40  // numbers per transposed row: 32 keys and 8 spare
+
+template <int NW, int NR, bool DEC>  // rank + rot_dim <= 32 NW, rank <= 16 NR
+__global__ void __launch_bounds__(256)
+latent_attn_mfma_kernel(const __bf16* __restrict__ ql, int64_t ql_t, int64_t ql_h, const __bf16* __restrict__ qr,
+                        int64_t qr_t, int64_t qr_h, const __bf16* __restrict__ cache,
+                        const int32_t* __restrict__ block_table, const int32_t* __restrict__ seq_of_token,
+                        const int32_t* __restrict__ positions, __bf16* __restrict__ out, int64_t out_t, int64_t out_h,
+                        float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits, int tokens, int heads,
+                        int rank, int rot_dim, int page_size, int max_blocks, float scale_log2, int n_tiles) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char latm_lds[];
+  constexpr int NP = (4 * NW + 7) / 8;  // 16-byte pieces of a round's rows that a thread moves
+  const int width = rank + rot_dim, kstride = width + LATM_KPAD;
+  const int p8 = width / 8, pieces = LATM_KEYS * p8;
+  const int nw = width / 32, nr = rank / 16;
+  __bf16* k_s = reinterpret_cast<__bf16*>(latm_lds);  // [32][kstride]
+  __bf16* vt_s = k_s + LATM_KEYS * kstride;            // [rank][LATM_VSTRIDE]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  int row, head, r0, r1;
+  bool wave_on;
+  if constexpr (DEC) {
+    r0 = blockIdx.x;
+    r1 = r0 + 1;
+    row = r0;
+    head = (blockIdx.y * 4 + wave) * 16 + n;
+    wave_on = (blockIdx.y * 4 + wave) * 16 < heads;
+  } else {
+    r0 = (n_tiles - 1 - static_cast<int>(blockIdx.x)) * 16;  // the tiles with the most keys start first
+    r1 = min(r0 + 16, tokens);
+    row = r0 + n;
+    head = blockIdx.y * 4 + wave;
+    wave_on = head < heads;
+  }
+  const bool col_ok = row < r1 && head < heads;
+
+  lat_bf16x8 qf[NW];
+#pragma unroll
+  for (int s = 0; s < NW; ++s) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<__bf16>(0.f);
+    if (s < nw && col_ok) {
+      const int i = 32 * s + 8 * g;
+      const __bf16* src = i < rank ? ql + row * ql_t + head * ql_h + i : qr + row * qr_t + head * qr_h + (i - rank);
+      qf[s] = *reinterpret_cast<const lat_bf16x8*>(src);
+    }
+  }
+  lat_f32x4 acc[NR];
+#pragma unroll
+  for (int d = 0; d < NR; ++d) acc[d] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -1e30f, l = 0.f;
+  const int ka0 = 8 * (n >> 2) + (n & 3), ka1 = ka0 + 4;  // the keys of this lane's rows of the two A operands
+
+  int seg = r0;
+  while (seg < r1) {  // (every decision in this loop is the same for the whole workgroup)
+    const int seq = seq_of_token[seg];
+    int end = seg + 1;
+    if constexpr (!DEC)
+      while (end < r1 && seq_of_token[end] == seq) ++end;
+    int k_begin = 0, k_end = positions[end - 1] + 1;  // a request's rows come in the order of their positions
+    if constexpr (DEC) {
+      const int per = ((k_end + n_splits - 1) / n_splits + LATM_KEYS - 1) & ~(LATM_KEYS - 1);
+      k_begin = static_cast<int>(blockIdx.z) * per;
+      k_end = min(k_end, k_begin + per);
+    }
+    const int my_pos = (col_ok && row >= seg && row < end) ? positions[row] : -1;
+    const int32_t* table = block_table + static_cast<int64_t>(seq) * max_blocks;
+
+    uint4 st[NP];
+    auto ask = [&](int k0) {
+#pragma unroll
+      for (int u = 0; u < NP; ++u) {
+        const int id = u * 256 + tid;
+        const int kk = id / p8, pc = id - kk * p8, j = k0 + kk;
+        st[u] = uint4{0u, 0u, 0u, 0u};  // rows past the last key enter LDS as zeros
+        if (id < pieces && j < k_end) {
+          const int64_t at = (static_cast<int64_t>(table[j / page_size]) * page_size + j % page_size) * width;
+          st[u] = *reinterpret_cast<const uint4*>(cache + at + 8 * pc);
+        }
+      }
+    };
+    auto put = [&]() {
+#pragma unroll
+      for (int u = 0; u < NP; ++u) {
+        const int id = u * 256 + tid;
+        if (id < pieces) {
+          const int kk = id / p8, pc = id - kk * p8;
+          *reinterpret_cast<uint4*>(k_s + kk * kstride + 8 * pc) = st[u];
+          if (8 * pc < rank) {
+            unsigned short* dst = reinterpret_cast<unsigned short*>(vt_s) + (8 * pc) * LATM_VSTRIDE + kk;
+            const unsigned int w[4] = {st[u].x, st[u].y, st[u].z, st[u].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              dst[(2 * e) * LATM_VSTRIDE] = static_cast<unsigned short>(w[e] & 0xffffu);
+              dst[(2 * e + 1) * LATM_VSTRIDE] = static_cast<unsigned short>(w[e] >> 16);
+            }
+          }
+        }
+      }
+    };
+
+    if (k_begin < k_end) {
+      ask(k_begin);
+      for (int k0 = k_begin; k0 < k_end; k0 += LATM_KEYS) {
+        __syncthreads();  // the round before has been read
+        put();
+        __syncthreads();
+        if (k0 + LATM_KEYS < k_end) ask(k0 + LATM_KEYS);
+        if (!wave_on) continue;
+        lat_f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NW; ++s) {
+          if (s < nw) {
+            const lat_bf16x8 a0 = *reinterpret_cast<const lat_bf16x8*>(k_s + ka0 * kstride + 32 * s + 8 * g);
+            const lat_bf16x8 a1 = *reinterpret_cast<const lat_bf16x8*>(k_s + ka1 * kstride + 32 * s + 8 * g);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[s], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[s], s1, 0, 0, 0);
+          }
+        }
+        float p[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = k0 + 8 * g + i;
+          p[i] = (j <= my_pos && j < k_end) ? s0[i] * scale_log2 : -INFINITY;
+          p[4 + i] = (j + 4 <= my_pos && j + 4 < k_end) ? s1[i] * scale_log2 : -INFINITY;
+          mx = fmaxf(mx, fmaxf(p[i], p[4 + i]));
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m, mx);
+        const float alpha = exp2f(m - m_new);
+        m = m_new;
+        float sum = 0.f;
+        lat_bf16x8 pb;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          p[i] = exp2f(p[i] - m_new);
+          sum += p[i];
+          pb[i] = static_cast<__bf16>(p[i]);
+        }
+        l = l * alpha + sum;
+        const bool rescale = !__all(alpha == 1.0f);
+#pragma unroll
+        for (int d = 0; d < NR; ++d) {
+          if (d < nr) {
+            if (rescale) acc[d] *= alpha;
+            const lat_bf16x8 a = *reinterpret_cast<const lat_bf16x8*>(vt_s + (16 * d + n) * LATM_VSTRIDE + 8 * g);
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[d], 0, 0, 0);
+          }
+        }
+      }
+    }
+    seg = end;
+  }
+
+  if (!wave_on) return;
+  float lt = l + __shfl_xor(l, 16);
+  lt += __shfl_xor(lt, 32);
+  if (!col_ok) return;
+  if (DEC && n_splits > 1) {
+    const int64_t p = (static_cast<int64_t>(row) * heads + head) * n_splits + blockIdx.z;
+#pragma unroll
+    for (int d = 0; d < NR; ++d)
+      if (d < nr) *reinterpret_cast<lat_f32x4*>(part_o + p * rank + 16 * d + 4 * g) = acc[d];
+    if (g == 0) {
+      part_ml[2 * p] = lt > 0.f ? m : -INFINITY;
+      part_ml[2 * p + 1] = lt;
+    }
+  } else {
+    const float inv = 1.0f / lt;
+#pragma unroll
+    for (int d = 0; d < NR; ++d) {
+      if (d < nr) {
+        lat_bf16x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = static_cast<__bf16>(acc[d][i] * inv);
+        *reinterpret_cast<lat_bf16x4*>(out + row * out_t + head * out_h + 16 * d + 4 * g) = o;
+      }
+    }
+  }
+}
+
+// decode != 0: one token per request (tokens == requests); with n_splits > 1 the keys are cut into that many slices,
+// part_o float32 [tokens * heads * n_splits, rank] and part_ml float32 [tokens * heads * n_splits, 2] take what the
+// slices leave, and out must be contiguous [tokens, heads, rank].
+extern "C" int ix_latent_attention_mfma(const void* ql, int64_t ql_t, int64_t ql_h, const void* qr, int64_t qr_t,
+                                        int64_t qr_h, const void* cache, const int32_t* block_table,
+                                        const int32_t* seq_of_token, const int32_t* positions, void* out,
+                                        int64_t out_t, int64_t out_h, float* part_o, float* part_ml, int n_splits,
+                                        int64_t tokens, int heads, int rank, int rot_dim, int page_size,
+                                        int max_blocks, float scale, int decode, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && tokens < (1 << 30) && heads > 0 && rank > 0 && rot_dim >= 0 && page_size > 0 && max_blocks > 0,
+             "sizes must be positive");
+  const int width = rank + rot_dim;
+  IX_REQUIRE(width % 32 == 0 && rank % 16 == 0 && width <= 576 && rank <= 512,
+             "rank + rot_dim must be a multiple of 32 up to 576, rank a multiple of 16 up to 512");
+  IX_REQUIRE(((reinterpret_cast<uintptr_t>(ql) | reinterpret_cast<uintptr_t>(qr) | reinterpret_cast<uintptr_t>(cache)) & 15) == 0 &&
+                 (ql_t | ql_h | qr_t | qr_h) % 8 == 0 && (rot_dim == 0 || rank % 8 == 0),
+             "queries and cache must lie on 16-byte boundaries");
+  IX_REQUIRE((reinterpret_cast<uintptr_t>(out) & 7) == 0 && (out_t | out_h) % 4 == 0, "out must lie on 8-byte boundaries");
+  IX_REQUIRE(n_splits >= 1 && n_splits <= 256 && (decode || n_splits == 1), "1 to 256 slices, and only for single tokens");
+  IX_REQUIRE(n_splits == 1 || (part_o != nullptr && part_ml != nullptr && out_h == rank && out_t == static_cast<int64_t>(heads) * rank),
+             "slices need their workspace and a contiguous result");
+  IX_REQUIRE(heads < 65536 * 4, "too many heads for one launch");
+  if (tokens == 0) return 0;
+  const int n_tiles = static_cast<int>((tokens + 15) / 16);
+  const size_t lds = (static_cast<size_t>(LATM_KEYS) * (width + LATM_KPAD) + static_cast<size_t>(rank) * LATM_VSTRIDE) * 2;
+  const dim3 grid = decode ? dim3(static_cast<unsigned>(tokens), (heads + 63) / 64, n_splits)
+                           : dim3(static_cast<unsigned>(n_tiles), (heads + 3) / 4, 1);
+  const float scale_log2 = scale * 1.4426950408889634f;
+#define LAUNCH(NW, NR, DEC)                                                                                             \
+  do {                                                                                                                  \
+    auto kernel = latent_attn_mfma_kernel<NW, NR, DEC>;                                                                 \
+    if (lds > 48 * 1024) {                                                                                              \
+      static bool raised = false;                                                                                       \
+      if (!raised) {                                                                                                    \
+        /* (a refusal shows as the launch's own error) */                                                              \
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,    \
+                                  96 * 1024);                                                                           \
+        (void)hipGetLastError();                                                                                        \
+        raised = true;                                                                                                  \
+      }                                                                                                                 \
+    }                                                                                                                   \
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, (const __bf16*)ql, ql_t, ql_h, (const __bf16*)qr, qr_t,     \
+                       qr_h, (const __bf16*)cache, block_table, seq_of_token, positions, (__bf16*)out, out_t, out_h,     \
+                       part_o, part_ml, n_splits, static_cast<int>(tokens), heads, rank, rot_dim, page_size, max_blocks, \
+                       scale_log2, n_tiles);                                                                            \
+  } while (0)
+#define BY_SIZE(DEC)                                        \
+  if (width <= 128 && rank <= 128) LAUNCH(4, 8, DEC);       \
+  else if (width <= 320 && rank <= 256) LAUNCH(10, 16, DEC); \
+  else LAUNCH(18, 32, DEC)
+  if (decode) { BY_SIZE(true); } else { BY_SIZE(false); }
+#undef BY_SIZE
+#undef LAUNCH
+  if (ix_check_launch("ix_latent_attention_mfma")) return 1;
+  if (n_splits > 1) return ix_attention_combine(part_o, part_ml, out, tokens, heads, n_splits, rank, stream);
+  return 0;
+}

@@ -85,6 +85,199 @@ linear_state_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* _
   }
 }
 
+// The same recurrence for requests that bring many rows (prompt portions).  The operands of a row are the same for
+// every column of a head, so a workgroup of four wavefronts shares them: it brings LS_CHUNK rows of r and k (and of
+// w, a, b) into LDS at a time, as float32 and through silu where asked, all loads of a chunk in flight at once and a
+// chunk ahead of the arithmetic.  SP lanes share a column (RPL = dim / SP rows each, in registers), so a workgroup
+// owns 256 / SP columns, and a row costs a lane five (or two) reads of RPL numbers from LDS, three sweeps over
+// them and two sums over SP lanes.  CORR: w, a, b come per row and channel; else the decay is one number per head.
+#define LS_CHUNK 16
+#define LS_THREADS 256
+
+template <int SP>
+__device__ __forceinline__ float ls_sum_over(float x) {  // over the SP neighbouring lanes of a column
+  x += ix_dpp<IX_DPP_XOR1>(x);
+  x += ix_dpp<IX_DPP_XOR2>(x);
+  if constexpr (SP >= 8) x += ix_dpp<IX_DPP_HALF_MIRROR>(x);
+  if constexpr (SP >= 16) x += ix_dpp<IX_DPP_MIRROR>(x);
+  return x;
+}
+
+__device__ __forceinline__ void ls_load8(const float* p, float (&o)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+__device__ __forceinline__ void ls_load8(const bf16_t* p, float (&o)[8]) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  o[0] = __uint_as_float(a.x << 16); o[1] = __uint_as_float(a.x & 0xffff0000u);
+  o[2] = __uint_as_float(a.y << 16); o[3] = __uint_as_float(a.y & 0xffff0000u);
+  o[4] = __uint_as_float(a.z << 16); o[5] = __uint_as_float(a.z & 0xffff0000u);
+  o[6] = __uint_as_float(a.w << 16); o[7] = __uint_as_float(a.w & 0xffff0000u);
+}
+
+template <typename T, int SP, int RPL, bool CORR>
+__global__ void __launch_bounds__(LS_THREADS)
+linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, int64_t r_stride,
+                          int64_t k_stride, int64_t v_stride, const float* __restrict__ w_rows,
+                          const float* __restrict__ w_head, const float* __restrict__ a_rows,
+                          const float* __restrict__ b_rows, float* __restrict__ state, int64_t state_stride,
+                          const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
+                          float* __restrict__ out, int heads, int vdim, int silu) {
+  constexpr int DIM = SP * RPL;
+  constexpr int COLS = LS_THREADS / SP;                 // value columns of a workgroup
+  constexpr int P8 = DIM / 8, P4 = DIM / 4;             // pieces of a row: of eight numbers (r, k), of four (w, a, b)
+  constexpr int RK_PIECES = LS_CHUNK * 2 * P8;
+  constexpr int RK_PER = (RK_PIECES + LS_THREADS - 1) / LS_THREADS;
+  constexpr int WAB_PIECES = CORR ? LS_CHUNK * 3 * P4 : 0;
+  constexpr int WAB_PER = CORR ? (WAB_PIECES + LS_THREADS - 1) / LS_THREADS : 1;
+  constexpr int V_PER = (LS_CHUNK * COLS + LS_THREADS - 1) / LS_THREADS;
+  __shared__ float4 rk_s[LS_CHUNK][2][P4];              // [row][k, r]
+  __shared__ float4 wab_s[CORR ? LS_CHUNK : 1][3][P4];  // [row][w, a, b]
+  __shared__ float v_s[LS_CHUNK][COLS];
+  const int tid = threadIdx.x;
+  const int col0 = blockIdx.x * COLS;
+  const int col = col0 + tid / SP, part = tid % SP;
+  const int head = blockIdx.y, seq = blockIdx.z;
+  const int64_t row0 = q_start[seq];
+  const int n = q_start[seq + 1] - static_cast<int>(row0);
+  if (n <= 0) return;
+  const bool live = col < vdim;
+  const int cj = live ? col : vdim - 1;  // lanes past the last column repeat it and store nothing
+  float* sp = state + static_cast<int64_t>(state_slots[seq]) * state_stride +
+              (static_cast<int64_t>(head) * vdim + cj) * DIM + part * RPL;
+  float S[RPL];
+#pragma unroll
+  for (int i = 0; i < RPL; i += 4) {
+    const float4 x = *reinterpret_cast<const float4*>(sp + i);
+    S[i] = x.x; S[i + 1] = x.y; S[i + 2] = x.z; S[i + 3] = x.w;
+  }
+  const float wh = CORR ? 1.0f : w_head[head];
+  const int64_t chan = static_cast<int64_t>(heads) * DIM;  // channels of a row of w, a, b
+
+  float st_rk[RK_PER][8], st_v[V_PER];
+  float4 st_wab[WAB_PER];
+  auto ask = [&](int first) {  // rows first .. first + LS_CHUNK - 1 of the portion (rows past its end repeat the last)
+#pragma unroll
+    for (int u = 0; u < RK_PER; ++u) {
+      const int id = min(u * LS_THREADS + tid, RK_PIECES - 1);
+      const int row = id / (2 * P8), which = (id / P8) & 1, pc = id % P8;
+      const int64_t at = row0 + min(first + row, n - 1);
+      ls_load8((which ? r + at * r_stride : k + at * k_stride) + head * DIM + 8 * pc, st_rk[u]);
+    }
+    if constexpr (CORR) {
+#pragma unroll
+      for (int u = 0; u < WAB_PER; ++u) {
+        const int id = min(u * LS_THREADS + tid, WAB_PIECES - 1);
+        const int row = id / (3 * P4), which = (id / P4) % 3, pc = id % P4;
+        const float* src = which == 0 ? w_rows : (which == 1 ? a_rows : b_rows);
+        st_wab[u] = *reinterpret_cast<const float4*>(src + (row0 + min(first + row, n - 1)) * chan + head * DIM + 4 * pc);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < V_PER; ++u) {
+      const int id = min(u * LS_THREADS + tid, LS_CHUNK * COLS - 1);
+      const int row = id / COLS, c = id % COLS;
+      st_v[u] = ix_load(v + (row0 + min(first + row, n - 1)) * v_stride + head * vdim + min(col0 + c, vdim - 1));
+    }
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int u = 0; u < RK_PER; ++u) {
+      const int id = u * LS_THREADS + tid;
+      if (id < RK_PIECES) {
+        const int row = id / (2 * P8), which = (id / P8) & 1, pc = id % P8;
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = silu ? ls_silu(st_rk[u][e]) : st_rk[u][e];
+        rk_s[row][which][2 * pc] = float4{x[0], x[1], x[2], x[3]};
+        rk_s[row][which][2 * pc + 1] = float4{x[4], x[5], x[6], x[7]};
+      }
+    }
+    if constexpr (CORR) {
+#pragma unroll
+      for (int u = 0; u < WAB_PER; ++u) {
+        const int id = u * LS_THREADS + tid;
+        if (id < WAB_PIECES) wab_s[id / (3 * P4)][(id / P4) % 3][id % P4] = st_wab[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < V_PER; ++u) {
+      const int id = u * LS_THREADS + tid;
+      if (id < LS_CHUNK * COLS) v_s[id / COLS][id % COLS] = silu ? ls_silu(st_v[u]) : st_v[u];
+    }
+  };
+  auto fetch = [&](int row, float4 (&kk)[RPL / 4], float4 (&rr)[RPL / 4], float4 (&ww)[RPL / 4], float4 (&aa)[RPL / 4],
+                   float4 (&bb)[RPL / 4], float& vv) {
+#pragma unroll
+    for (int j = 0; j < RPL / 4; ++j) {
+      kk[j] = rk_s[row][0][part * (RPL / 4) + j];
+      rr[j] = rk_s[row][1][part * (RPL / 4) + j];
+      if constexpr (CORR) {
+        ww[j] = wab_s[row][0][part * (RPL / 4) + j];
+        aa[j] = wab_s[row][1][part * (RPL / 4) + j];
+        bb[j] = wab_s[row][2][part * (RPL / 4) + j];
+      }
+    }
+    vv = v_s[row][tid / SP];
+  };
+
+  ask(0);
+  for (int first = 0; first < n; first += LS_CHUNK) {
+    __syncthreads();  // the chunk before has been read
+    put();
+    __syncthreads();
+    if (first + LS_CHUNK < n) ask(first + LS_CHUNK);  // on their way while this chunk is worked
+    __builtin_amdgcn_sched_barrier(0);
+    const int rows = min(LS_CHUNK, n - first);
+    float4 kc[RPL / 4], rc[RPL / 4], wc[RPL / 4], ac[RPL / 4], bc[RPL / 4];
+    float vc;
+    fetch(0, kc, rc, wc, ac, bc, vc);
+    for (int i = 0; i < rows; ++i) {
+      float4 kn[RPL / 4], rn[RPL / 4], wn[RPL / 4], an[RPL / 4], bn[RPL / 4];
+      float vn;
+      fetch(min(i + 1, LS_CHUNK - 1), kn, rn, wn, an, bn, vn);
+      float read = 0.f;
+      if constexpr (CORR) {
+#pragma unroll
+        for (int j = 0; j < RPL / 4; ++j)
+          read += bc[j].x * S[4 * j] + bc[j].y * S[4 * j + 1] + bc[j].z * S[4 * j + 2] + bc[j].w * S[4 * j + 3];
+        read = ls_sum_over<SP>(read);
+      }
+      float o = 0.f;
+#pragma unroll
+      for (int j = 0; j < RPL / 4; ++j) {
+        const float ke[4] = {kc[j].x, kc[j].y, kc[j].z, kc[j].w}, re[4] = {rc[j].x, rc[j].y, rc[j].z, rc[j].w};
+        const float we[4] = {wc[j].x, wc[j].y, wc[j].z, wc[j].w}, ae[4] = {ac[j].x, ac[j].y, ac[j].z, ac[j].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float& s = S[4 * j + e];
+          if constexpr (CORR) s = we[e] * s - ae[e] * read + ke[e] * vc;
+          else s = wh * s + ke[e] * vc;
+          o += re[e] * s;
+        }
+      }
+      o = ls_sum_over<SP>(o);
+      if (live && part == 0) out[((row0 + first + i) * heads + head) * vdim + col] = o;
+#pragma unroll
+      for (int j = 0; j < RPL / 4; ++j) {
+        kc[j] = kn[j];
+        rc[j] = rn[j];
+        if constexpr (CORR) {
+          wc[j] = wn[j];
+          ac[j] = an[j];
+          bc[j] = bn[j];
+        }
+      }
+      vc = vn;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < RPL; i += 4) *reinterpret_cast<float4*>(sp + i) = float4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+  }
+}
+
 extern "C" int ix_linear_state(const void* r, const void* k, const void* v, int dtype, int64_t r_stride,
                                int64_t k_stride, int64_t v_stride, const float* w_rows, const float* w_head,
                                const float* a_rows, const float* b_rows, float* state, int64_t state_stride,
@@ -97,6 +290,38 @@ extern "C" int ix_linear_state(const void* r, const void* k, const void* v, int 
   IX_REQUIRE(state_stride >= static_cast<int64_t>(heads) * dim * vdim, "a slot's state is too small");
   IX_REQUIRE(requests < 65536 && heads < 65536, "too many requests or heads for one launch");
   if (tokens == 0) return 0;
+  // steps that bring a request many rows: chunks through LDS, where a head's keys are 16 .. 128 numbers, the
+  // operands come in the two usual combinations, and every row starts on a 16-byte boundary
+  {
+    const int elt = dtype == IX_F32 ? 4 : 2;
+    const bool corr = w_rows != nullptr && a_rows != nullptr;
+    const bool none = w_head != nullptr && a_rows == nullptr;
+    const uintptr_t all = reinterpret_cast<uintptr_t>(r) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(state) |
+                          reinterpret_cast<uintptr_t>(w_rows) | reinterpret_cast<uintptr_t>(a_rows) |
+                          reinterpret_cast<uintptr_t>(b_rows);
+    const bool aligned = (all & 15) == 0 && (r_stride * elt) % 16 == 0 && (k_stride * elt) % 16 == 0 && state_stride % 4 == 0;
+    if ((dtype == IX_F32 || dtype == IX_BF16) && (corr || none) && aligned && tokens >= 4 * static_cast<int64_t>(requests) &&
+        (dim == 16 || dim == 32 || dim == 64 || dim == 128)) {
+#define CHUNKED(T, SP, RPL, CORR)                                                                                        \
+  hipLaunchKernelGGL((linear_state_chunk_kernel<T, SP, RPL, CORR>),                                                      \
+                     dim3((vdim + LS_THREADS / SP - 1) / (LS_THREADS / SP), heads, requests), dim3(LS_THREADS), 0, stream, \
+                     (const T*)r, (const T*)k, (const T*)v, r_stride, k_stride, v_stride, w_rows, w_head, a_rows, b_rows, \
+                     state, state_stride, q_start, state_slots, out, heads, vdim, silu)
+#define BY_DIM(T, CORR)                            \
+  if (dim == 16) CHUNKED(T, 4, 4, CORR);           \
+  else if (dim == 32) CHUNKED(T, 8, 4, CORR);      \
+  else if (dim == 64) CHUNKED(T, 16, 4, CORR);     \
+  else CHUNKED(T, 16, 8, CORR)
+      if (dtype == IX_F32) {
+        if (corr) { BY_DIM(float, true); } else { BY_DIM(float, false); }
+      } else {
+        if (corr) { BY_DIM(bf16_t, true); } else { BY_DIM(bf16_t, false); }
+      }
+#undef BY_DIM
+#undef CHUNKED
+      return ix_check_launch("ix_linear_state");
+    }
+  }
   dim3 grid((vdim + 15) / 16, heads, requests), block(64);
 #define LAUNCH(T, R)                                                                                               \
   hipLaunchKernelGGL((linear_state_kernel<T, R>), grid, block, 0, stream, (const T*)r, (const T*)k, (const T*)v,    \

@@ -1256,3 +1256,58 @@ def latent_attention_plain(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torc
           _ptr(cache), _i32(_dt(q_lat)), _ptr(block_table), _ptr(seq_of_token), _ptr(positions), out.data_ptr(),
           _i64(o_t), _i64(o_h), _i64(T), _i32(heads), _i32(rank), _i32(rot_dim), _i32(cache.shape[2]),
           _i32(block_table.shape[1]), _f32(scale), _stream())
+
+
+LATENT_MFMA_MAX_SPLITS = 32
+
+
+def latent_mfma_fits(q_lat: torch.Tensor, q_rot: torch.Tensor, out: torch.Tensor, rank: int, rot_dim: int) -> bool:
+    """Whether the matrix-core kernel takes these operands: bfloat16, rank + rot_dim a multiple of 32 up to 576, rank a
+    multiple of 16 up to 512, queries on 16-byte and results on 8-byte boundaries."""
+    width = rank + rot_dim
+    if q_lat.dtype != torch.bfloat16 or width % 32 or rank % 16 or width > 576 or rank > 512:
+        return False
+    if q_lat.stride(2) != 1 or out.stride(2) != 1 or (rot_dim and q_rot.stride(2) != 1):
+        return False
+    if (q_lat.data_ptr() | q_rot.data_ptr()) % 16 or out.data_ptr() % 8:
+        return False
+    return not ((q_lat.stride(0) | q_lat.stride(1) | q_rot.stride(0) | q_rot.stride(1)) % 8
+                or (out.stride(0) | out.stride(1)) % 4)
+
+
+def latent_mfma_splits(tokens: int, heads: int) -> int:
+    """Into how many slices a step of one token per request cuts every request's keys: enough workgroups for the
+    compute units, whatever the contexts (a captured step keeps its number)."""
+    return max(1, min(LATENT_MFMA_MAX_SPLITS, 256 // (tokens * (-(-heads // 64)))))
+
+
+def latent_attention_mfma(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
+                          seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, rank: int,
+                          rot_dim: int, scale: float, one_token_each: bool = False, n_splits: int = 1,
+                          work: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> None:
+    """`latent_attention_plain` on the matrix cores (see `latent_mfma_fits`).  `one_token_each`: every request brings
+    one token; its keys may then be cut into `n_splits` slices, with `work` = float32 ([T * heads * n_splits, rank],
+    [T * heads * n_splits, 2]) and a contiguous `out` [T, heads, rank]."""
+    T, heads = q_lat.shape[0], q_lat.shape[1]
+    ql_t, ql_h = _head_rows(q_lat, T, heads, rank, "q_lat")
+    qr_t, qr_h = _head_rows(q_rot, T, heads, rot_dim, "q_rot")
+    o_t, o_h = _head_rows(out, T, heads, rank, "out")
+    _need(latent_mfma_fits(q_lat, q_rot, out, rank, rot_dim), "sizes or alignment that the matrix-core kernel does not take")
+    _need(q_rot.dtype == q_lat.dtype and out.dtype == q_lat.dtype and cache.dtype == q_lat.dtype, "one element type")
+    _need(cache.dim() == 4 and cache.shape[1] == 1 and cache.shape[3] == rank + rot_dim and cache.is_contiguous(),
+          "the cache must be [pages, 1, page_size, rank + rot_dim]")
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    _is_i32(block_table)
+    _is_i32(seq_of_token, T)
+    _is_i32(positions, T)
+    _need(n_splits == 1 or one_token_each, "keys are cut into slices for single tokens only")
+    part_o = part_ml = None
+    if n_splits > 1:
+        part_o, part_ml = work
+        _need(part_o.dtype == torch.float32 and part_o.numel() >= T * heads * n_splits * rank and part_o.is_contiguous()
+              and part_ml.dtype == torch.float32 and part_ml.numel() >= T * heads * n_splits * 2
+              and part_ml.is_contiguous() and out.is_contiguous(), "the slices' workspace or a result that is not contiguous")
+    _call("ix_latent_attention_mfma", q_lat.data_ptr(), _i64(ql_t), _i64(ql_h), q_rot.data_ptr(), _i64(qr_t), _i64(qr_h),
+          _ptr(cache), _ptr(block_table), _ptr(seq_of_token), _ptr(positions), out.data_ptr(), _i64(o_t), _i64(o_h),
+          _ptr(part_o), _ptr(part_ml), _i32(n_splits), _i64(T), _i32(heads), _i32(rank), _i32(rot_dim),
+          _i32(cache.shape[2]), _i32(block_table.shape[1]), _f32(scale), _i32(1 if one_token_each else 0), _stream())

@@ -84,15 +84,29 @@ class LatentAttention(Mixer):
                            ctx.slots[cache.group] if cache.writes else None, latent, H, self.rot_dim, self.kv_rank)
         q3 = q.unflatten(1, (H, self.q_dim))
         q_lat = torch.bmm(q3[:, :, :self.head_dim].transpose(0, 1), self.w_uk)  # [H, T, rank]
-        o_lat = rt.empty((H, T, self.kv_rank))
+        if ctx.one_token_each:  # (the slices of a token's keys meet in a contiguous [T, H, rank])
+            o_lat = rt.empty((T, H, self.kv_rank)).transpose(0, 1)
+        else:
+            o_lat = rt.empty((H, T, self.kv_rank))
         self.attend(ctx, q_lat.transpose(0, 1), q3[:, :, self.head_dim:], cache, o_lat.transpose(0, 1))
         y = rt.empty((T, H * self.value_dim))
         torch.bmm(o_lat, self.w_uv_t, out=y.view(T, H, self.value_dim).transpose(0, 1))
         return rt.linear(y, self.w_out)
 
     def attend(self, ctx, q_lat, q_rot, cache, out) -> None:
-        ops.latent_attention_plain(q_lat, q_rot, cache.arrays["latent"], ctx.block_tables[cache.group],
-                                   ctx.seq_of_token, ctx.positions, out, self.kv_rank, self.rot_dim, self.scale)
+        latent, table = cache.arrays["latent"], ctx.block_tables[cache.group]
+        if not ops.latent_mfma_fits(q_lat, q_rot, out, self.kv_rank, self.rot_dim):  # float32 runs, other sizes
+            ops.latent_attention_plain(q_lat, q_rot, latent, table, ctx.seq_of_token, ctx.positions, out, self.kv_rank,
+                                       self.rot_dim, self.scale)
+            return
+        rt, T, H = ctx.rt, q_lat.shape[0], self.num_heads
+        splits, work = 1, None
+        if ctx.one_token_each:
+            splits = ops.latent_mfma_splits(T, H)
+            if splits > 1:
+                work = (rt.empty((T * H * splits, self.kv_rank), torch.float32), rt.empty((T * H * splits, 2), torch.float32))
+        ops.latent_attention_mfma(q_lat, q_rot, latent, table, ctx.seq_of_token, ctx.positions, out, self.kv_rank,
+                                  self.rot_dim, self.scale, ctx.one_token_each, splits, work)
 
 
 register_part("mixer", "latent_attention", LatentAttention)

@@ -30,6 +30,17 @@ def bfloat16(x):
 _S = exact  # what keeping an activation between two operations does to it (`forward(store=...)` sets it)
 
 
+def jittered(seed):
+    """Another sample of what 16-bit storage does: x moved by up to one part in 512 at random (as much as the rounding itself), then rounded to
+    bfloat16.  (An engine rounds at other places than this model; several samples show better how far rounding alone
+    can move a badly conditioned position.)"""
+    g = torch.Generator().manual_seed(seed)
+
+    def store(x):
+        return bfloat16(x * (1.0 + (torch.rand(x.shape, generator=g, dtype=F) * 2.0 - 1.0) / 512.0))
+    return store
+
+
 def rms_unit(x, eps):
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
 

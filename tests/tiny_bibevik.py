@@ -80,7 +80,17 @@ E = config(77, 90, 1e-5, 1.0, [
     delta(2, 24, 4, experts(28, 1.0, 3, 1, 3.0, (1, 1))),
 ])
 del E["embedding"]
-CONFIGS = {"A": A, "B": B, "C": C, "D": D, "E": E}
+# F: sizes that the matrix-core attention and the chunked recurrence take (latents and rotated parts in multiples of
+# 16 and 32, heads of 32 and 64 numbers), two latent layers of different classes of size, one of them run twice
+_f0 = latent(4, 16, 32, 24, 32, 0.2, (32, 10000.0), dense(48, 1.0))
+F = config(200, 64, 1e-6, 3.0, [
+    _f0,
+    delta(2, 32, 4, experts(24, 1.0, 4, 2, 1.5, (2, 1), (16, 1.0))),
+    latent(2, 24, 64, 16, 128, 0.12, (48, 300.0), None),
+    lightning(2, 64, 32, [0.9, 0.99], dense(40, 1.5)),
+    again(_f0, 0),
+])
+CONFIGS = {"A": A, "B": B, "C": C, "D": D, "E": E, "F": F}
 
 
 def make_folder(raw_config: dict, seed: int, out_dir: str, dtype: str = "bfloat16") -> str:
