@@ -214,8 +214,12 @@ latent_attn_mfma_kernel(const __bf16* __restrict__ ql, int64_t ql_t, int64_t ql_
                         int rank, int rot_dim, int page_size, int max_blocks, float scale_log2, int n_tiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char latm_lds[];
   constexpr int NP = (4 * NW + 7) / 8;  // 16-byte pieces of a round's rows that a thread moves
-  const int width = rank + rot_dim, kstride = width + LATM_KPAD;
-  const int p8 = width / 8, pieces = LATM_KEYS * p8;
+  const int width = rank + rot_dim;
+  const int kstride = ((width + 63) & ~63) + LATM_KPAD;
+  // 16-byte piece p of key row r lies at place p ^ 4 for rows 8..15 and 24..31: the sixteen rows that one product
+  // reads at one piece index (0-3, 8-11, 16-19, 24-27, or the four after each) then fall on all banks evenly
+  auto key_place = [&](int r, int piece) { return r * kstride + ((piece ^ (((r >> 3) & 1) << 2)) << 3); };
+  const int p8 = width / 8;
   const int nw = width / 32, nr = rank / 16;
   __bf16* k_s = reinterpret_cast<__bf16*>(latm_lds);  // [32][kstride]
   __bf16* vt_s = k_s + LATM_KEYS * kstride;            // [rank][LATM_VSTRIDE]
@@ -231,10 +235,12 @@ latent_attn_mfma_kernel(const __bf16* __restrict__ ql, int64_t ql_t, int64_t ql_
     head = (blockIdx.y * 4 + wave) * 16 + n;
     wave_on = (blockIdx.y * 4 + wave) * 16 < heads;
   } else {
-    r0 = (n_tiles - 1 - static_cast<int>(blockIdx.x)) * 16;  // the tiles with the most keys start first
+    // one row of workgroups, the tiles with the most keys first, a tile's groups of four heads side by side
+    const int head_groups = (heads + 3) / 4;
+    r0 = (n_tiles - 1 - static_cast<int>(blockIdx.x) / head_groups) * 16;
     r1 = min(r0 + 16, tokens);
     row = r0 + n;
-    head = blockIdx.y * 4 + wave;
+    head = (static_cast<int>(blockIdx.x) % head_groups) * 4 + wave;
     wave_on = head < heads;
   }
   const bool col_ok = row < r1 && head < heads;
@@ -272,33 +278,41 @@ latent_attn_mfma_kernel(const __bf16* __restrict__ ql, int64_t ql_t, int64_t ql_
     const int32_t* table = block_table + static_cast<int64_t>(seq) * max_blocks;
 
     uint4 st[NP];
+    const int my_key = tid >> 3, my_sub = tid & 7;  // a thread moves pieces my_sub, my_sub + 8, .. of one key's row
     auto ask = [&](int k0) {
+      const int j = k0 + my_key;
+      const bool there = j < k_end;
+      const int64_t at = there ? (static_cast<int64_t>(table[j / page_size]) * page_size + j % page_size) * width : 0;
 #pragma unroll
       for (int u = 0; u < NP; ++u) {
-        const int id = u * 256 + tid;
-        const int kk = id / p8, pc = id - kk * p8, j = k0 + kk;
+        const int pc = my_sub + 8 * u;
         st[u] = uint4{0u, 0u, 0u, 0u};  // rows past the last key enter LDS as zeros
-        if (id < pieces && j < k_end) {
-          const int64_t at = (static_cast<int64_t>(table[j / page_size]) * page_size + j % page_size) * width;
-          st[u] = *reinterpret_cast<const uint4*>(cache + at + 8 * pc);
-        }
+        if (there && pc < p8) st[u] = *reinterpret_cast<const uint4*>(cache + at + 8 * pc);
       }
     };
     auto put = [&]() {
 #pragma unroll
       for (int u = 0; u < NP; ++u) {
-        const int id = u * 256 + tid;
-        if (id < pieces) {
-          const int kk = id / p8, pc = id - kk * p8;
-          *reinterpret_cast<uint4*>(k_s + kk * kstride + 8 * pc) = st[u];
-          if (8 * pc < rank) {
-            unsigned short* dst = reinterpret_cast<unsigned short*>(vt_s) + (8 * pc) * LATM_VSTRIDE + kk;
-            const unsigned int w[4] = {st[u].x, st[u].y, st[u].z, st[u].w};
+        const int pc = my_sub + 8 * u;
+        if (pc < p8) *reinterpret_cast<uint4*>(k_s + key_place(my_key, pc)) = st[u];
+      }
+    };
+    // The latent part once more, transposed, from the rows in LDS: here neighbouring lanes take neighbouring keys of
+    // the same eight numbers, so that their 2-byte writes fall side by side into a transposed row (lanes that
+    // held neighbouring pieces of one key would all write to the same bank).
+    auto turn = [&]() {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              dst[(2 * e) * LATM_VSTRIDE] = static_cast<unsigned short>(w[e] & 0xffffu);
-              dst[(2 * e + 1) * LATM_VSTRIDE] = static_cast<unsigned short>(w[e] >> 16);
-            }
+      for (int u = 0; u < (NR + 3) / 4; ++u) {
+        const int id = u * 256 + tid;
+        const int kk = id & (LATM_KEYS - 1), pc = id / LATM_KEYS;
+        if (8 * pc < rank) {
+          const uint4 x = *reinterpret_cast<const uint4*>(k_s + key_place(kk, pc));
+          unsigned short* dst = reinterpret_cast<unsigned short*>(vt_s) + (8 * pc) * LATM_VSTRIDE + kk;
+          const unsigned int w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            dst[(2 * e) * LATM_VSTRIDE] = static_cast<unsigned short>(w[e] & 0xffffu);
+            dst[(2 * e + 1) * LATM_VSTRIDE] = static_cast<unsigned short>(w[e] >> 16);
           }
         }
       }
@@ -310,14 +324,16 @@ latent_attn_mfma_kernel(const __bf16* __restrict__ ql, int64_t ql_t, int64_t ql_
         __syncthreads();  // the round before has been read
         put();
         __syncthreads();
+        turn();
+        __syncthreads();
         if (k0 + LATM_KEYS < k_end) ask(k0 + LATM_KEYS);
         if (!wave_on) continue;
         lat_f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < NW; ++s) {
           if (s < nw) {
-            const lat_bf16x8 a0 = *reinterpret_cast<const lat_bf16x8*>(k_s + ka0 * kstride + 32 * s + 8 * g);
-            const lat_bf16x8 a1 = *reinterpret_cast<const lat_bf16x8*>(k_s + ka1 * kstride + 32 * s + 8 * g);
+            const lat_bf16x8 a0 = *reinterpret_cast<const lat_bf16x8*>(k_s + key_place(ka0, 4 * s + g));
+            const lat_bf16x8 a1 = *reinterpret_cast<const lat_bf16x8*>(k_s + key_place(ka1, 4 * s + g));
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[s], s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[s], s1, 0, 0, 0);
           }
@@ -410,9 +426,9 @@ extern "C" int ix_latent_attention_mfma(const void* ql, int64_t ql_t, int64_t ql
   IX_REQUIRE(heads < 65536 * 4, "too many heads for one launch");
   if (tokens == 0) return 0;
   const int n_tiles = static_cast<int>((tokens + 15) / 16);
-  const size_t lds = (static_cast<size_t>(LATM_KEYS) * (width + LATM_KPAD) + static_cast<size_t>(rank) * LATM_VSTRIDE) * 2;
+  const size_t lds = (static_cast<size_t>(LATM_KEYS) * (((width + 63) & ~63) + LATM_KPAD) + static_cast<size_t>(rank) * LATM_VSTRIDE) * 2;
   const dim3 grid = decode ? dim3(static_cast<unsigned>(tokens), (heads + 63) / 64, n_splits)
-                           : dim3(static_cast<unsigned>(n_tiles), (heads + 3) / 4, 1);
+                           : dim3(static_cast<unsigned>(n_tiles) * ((heads + 3) / 4), 1, 1);
   const float scale_log2 = scale * 1.4426950408889634f;
 #define LAUNCH(NW, NR, DEC)                                                                                             \
   do {                                                                                                                  \
