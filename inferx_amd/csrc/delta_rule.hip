@@ -433,6 +433,38 @@ head_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ x2,
   }
 }
 
+// The same for wide rows (one norm over all heads' columns together: hundreds or thousands of numbers): a
+// workgroup per (token, head), so that a row's numbers are in flight at once instead of sixty-four at a time.
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_norm_gate_wide_kernel(const float* __restrict__ x, const float* __restrict__ x2, float lambda,
+                           const void* __restrict__ weight, int w_dtype, const T* __restrict__ gate,
+                           int64_t gate_stride, T* __restrict__ out, int heads, int vdim, float eps, float mult,
+                           int weight_per_head, int gate_sigmoid) {
+  __shared__ float red[16];
+  const int64_t p = blockIdx.x;
+  const int64_t t = p / heads;
+  const int head = static_cast<int>(p % heads);
+  const float* xr = x + p * vdim;
+  const float* x2r = x2 ? x2 + p * vdim : nullptr;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < vdim; j += 256) {
+    const float o = x2r ? xr[j] - lambda * x2r[j] : xr[j];
+    ss += o * o;
+  }
+  ss = ix_block_sum(ss, red);
+  const float inv = mult / sqrtf(ss / static_cast<float>(vdim) + eps);
+  for (int j = threadIdx.x; j < vdim; j += 256) {
+    float y = (x2r ? xr[j] - lambda * x2r[j] : xr[j]) * inv;
+    if (weight) y *= ix_load_rt(weight, w_dtype, weight_per_head ? head * vdim + j : j);
+    if (gate) {
+      const float gv = ix_load(gate + t * gate_stride + head * vdim + j);
+      y *= (gate_sigmoid ? 1.0f : gv) / (1.0f + expf(-gv));
+    }
+    ix_store(out + p * vdim + j, y);
+  }
+}
+
 extern "C" int ix_head_norm_gate(const float* x, const float* x2, float lambda, const void* weight, int w_dtype,
                                  const void* gate, int64_t gate_stride, void* out, int dtype, int64_t tokens,
                                  int heads, int vdim, float eps, float mult, int weight_per_head, int gate_sigmoid,
@@ -442,6 +474,19 @@ extern "C" int ix_head_norm_gate(const float* x, const float* x2, float lambda, 
   if (tokens == 0) return 0;
   const int64_t pairs = tokens * heads;
   IX_REQUIRE((pairs + 3) / 4 < (1ll << 31), "too many rows for one launch");
+  if (vdim >= 512) {
+    IX_REQUIRE(pairs < (1ll << 31), "too many rows for one launch");
+    dim3 wide(static_cast<unsigned>(pairs)), threads(256);
+    if (dtype == IX_F32)
+      hipLaunchKernelGGL(head_norm_gate_wide_kernel<float>, wide, threads, 0, stream, x, x2, lambda, weight, w_dtype,
+                         (const float*)gate, gate_stride, (float*)out, heads, vdim, eps, mult, weight_per_head,
+                         gate_sigmoid);
+    else
+      hipLaunchKernelGGL(head_norm_gate_wide_kernel<bf16_t>, wide, threads, 0, stream, x, x2, lambda, weight, w_dtype,
+                         (const bf16_t*)gate, gate_stride, (bf16_t*)out, heads, vdim, eps, mult, weight_per_head,
+                         gate_sigmoid);
+    return ix_check_launch("ix_head_norm_gate");
+  }
   dim3 grid(static_cast<unsigned>((pairs + 3) / 4)), block(256);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, x, x2, lambda, weight, w_dtype,

@@ -22,8 +22,22 @@ __device__ __forceinline__ float ls_quad_sum(float v) {
 
 __device__ __forceinline__ float ls_silu(float x) { return x / (1.0f + expf(-x)); }
 
-// R: rows of a column per lane (4 R >= dim)
-template <typename T, int R>
+__device__ __forceinline__ void ls_load8(const float* p, float (&o)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+__device__ __forceinline__ void ls_load8(const bf16_t* p, float (&o)[8]) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  o[0] = __uint_as_float(a.x << 16); o[1] = __uint_as_float(a.x & 0xffff0000u);
+  o[2] = __uint_as_float(a.y << 16); o[3] = __uint_as_float(a.y & 0xffff0000u);
+  o[4] = __uint_as_float(a.z << 16); o[5] = __uint_as_float(a.z & 0xffff0000u);
+  o[6] = __uint_as_float(a.w << 16); o[7] = __uint_as_float(a.w & 0xffff0000u);
+}
+
+// R: rows of a column per lane (4 R >= dim).  VEC: dim = 4 R, R a multiple of 8 and everything on 16-byte boundaries,
+// so that a lane reads its part of the state and of every operand in 16-byte pieces.
+template <typename T, int R, bool VEC>
 __global__ void __launch_bounds__(64)
 linear_state_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, int64_t r_stride,
                     int64_t k_stride, int64_t v_stride, const float* __restrict__ w_rows,
@@ -41,12 +55,43 @@ linear_state_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* _
   float* sp = state + static_cast<int64_t>(state_slots[seq]) * state_stride +
               (static_cast<int64_t>(head) * vdim + (live ? col : 0)) * dim;
   float s[R];
+  if constexpr (VEC) {
 #pragma unroll
-  for (int i = 0; i < R; ++i) s[i] = (live && row0 + i < dim) ? sp[row0 + i] : 0.f;
+    for (int i = 0; i < R; i += 4) {
+      const float4 x = live ? *reinterpret_cast<const float4*>(sp + row0 + i) : float4{0.f, 0.f, 0.f, 0.f};
+      s[i] = x.x; s[i + 1] = x.y; s[i + 2] = x.z; s[i + 3] = x.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < R; ++i) s[i] = (live && row0 + i < dim) ? sp[row0 + i] : 0.f;
+  }
   const float wh = w_head ? w_head[head] : 1.0f;
   const int64_t ch = static_cast<int64_t>(head) * dim;  // first key channel of this head
   for (int t = t0; t < t1; ++t) {
     float rr[R], kk[R], ww[R], aa[R], bb[R];
+    if constexpr (VEC) {
+      const int64_t c = ch + row0, at = static_cast<int64_t>(t) * heads * dim + c;
+#pragma unroll
+      for (int i = 0; i < R; i += 8) {
+        float x[8], y[8];
+        ls_load8(r + t * r_stride + c + i, x);
+        ls_load8(k + t * k_stride + c + i, y);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          rr[i + e] = silu ? ls_silu(x[e]) : x[e];
+          kk[i + e] = silu ? ls_silu(y[e]) : y[e];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < R; i += 4) {
+        const float4 w4 = w_rows ? *reinterpret_cast<const float4*>(w_rows + at + i) : float4{wh, wh, wh, wh};
+        const float4 a4 = a_rows ? *reinterpret_cast<const float4*>(a_rows + at + i) : float4{0.f, 0.f, 0.f, 0.f};
+        const float4 b4 = b_rows ? *reinterpret_cast<const float4*>(b_rows + at + i) : float4{0.f, 0.f, 0.f, 0.f};
+        ww[i] = w4.x; ww[i + 1] = w4.y; ww[i + 2] = w4.z; ww[i + 3] = w4.w;
+        aa[i] = a4.x; aa[i + 1] = a4.y; aa[i + 2] = a4.z; aa[i + 3] = a4.w;
+        bb[i] = b4.x; bb[i + 1] = b4.y; bb[i + 2] = b4.z; bb[i + 3] = b4.w;
+      }
+    } else
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       const bool ok = row0 + i < dim;
@@ -79,9 +124,14 @@ linear_state_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* _
     if (live && part == 0) out[(static_cast<int64_t>(t) * heads + head) * vdim + col] = o;
   }
   if (live) {
+    if constexpr (VEC) {
 #pragma unroll
-    for (int i = 0; i < R; ++i)
-      if (row0 + i < dim) sp[row0 + i] = s[i];
+      for (int i = 0; i < R; i += 4) *reinterpret_cast<float4*>(sp + row0 + i) = float4{s[i], s[i + 1], s[i + 2], s[i + 3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+        if (row0 + i < dim) sp[row0 + i] = s[i];
+    }
   }
 }
 
@@ -101,19 +151,6 @@ __device__ __forceinline__ float ls_sum_over(float x) {  // over the SP neighbou
   if constexpr (SP >= 8) x += ix_dpp<IX_DPP_HALF_MIRROR>(x);
   if constexpr (SP >= 16) x += ix_dpp<IX_DPP_MIRROR>(x);
   return x;
-}
-
-__device__ __forceinline__ void ls_load8(const float* p, float (&o)[8]) {
-  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
-  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
-  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
-}
-__device__ __forceinline__ void ls_load8(const bf16_t* p, float (&o)[8]) {
-  const uint4 a = *reinterpret_cast<const uint4*>(p);
-  o[0] = __uint_as_float(a.x << 16); o[1] = __uint_as_float(a.x & 0xffff0000u);
-  o[2] = __uint_as_float(a.y << 16); o[3] = __uint_as_float(a.y & 0xffff0000u);
-  o[4] = __uint_as_float(a.z << 16); o[5] = __uint_as_float(a.z & 0xffff0000u);
-  o[6] = __uint_as_float(a.w << 16); o[7] = __uint_as_float(a.w & 0xffff0000u);
 }
 
 template <typename T, int SP, int RPL, bool CORR>
@@ -292,6 +329,7 @@ extern "C" int ix_linear_state(const void* r, const void* k, const void* v, int 
   if (tokens == 0) return 0;
   // steps that bring a request many rows: chunks through LDS, where a head's keys are 16 .. 128 numbers, the
   // operands come in the two usual combinations, and every row starts on a 16-byte boundary
+  bool vec16 = false;
   {
     const int elt = dtype == IX_F32 ? 4 : 2;
     const bool corr = w_rows != nullptr && a_rows != nullptr;
@@ -300,6 +338,7 @@ extern "C" int ix_linear_state(const void* r, const void* k, const void* v, int 
                           reinterpret_cast<uintptr_t>(w_rows) | reinterpret_cast<uintptr_t>(a_rows) |
                           reinterpret_cast<uintptr_t>(b_rows);
     const bool aligned = (all & 15) == 0 && (r_stride * elt) % 16 == 0 && (k_stride * elt) % 16 == 0 && state_stride % 4 == 0;
+    vec16 = aligned;
     if ((dtype == IX_F32 || dtype == IX_BF16) && (corr || none) && aligned && tokens >= 4 * static_cast<int64_t>(requests) &&
         (dim == 16 || dim == 32 || dim == 64 || dim == 128)) {
 #define CHUNKED(T, SP, RPL, CORR)                                                                                        \
@@ -323,16 +362,20 @@ extern "C" int ix_linear_state(const void* r, const void* k, const void* v, int 
     }
   }
   dim3 grid((vdim + 15) / 16, heads, requests), block(64);
-#define LAUNCH(T, R)                                                                                               \
-  hipLaunchKernelGGL((linear_state_kernel<T, R>), grid, block, 0, stream, (const T*)r, (const T*)k, (const T*)v,    \
-                     r_stride, k_stride, v_stride, w_rows, w_head, a_rows, b_rows, state, state_stride, q_start,    \
-                     state_slots, out, heads, dim, vdim, silu)
-#define PICK(T)                        \
-  if (dim <= 16) LAUNCH(T, 4);         \
-  else if (dim <= 32) LAUNCH(T, 8);    \
-  else if (dim <= 64) LAUNCH(T, 16);   \
-  else if (dim <= 128) LAUNCH(T, 32);  \
-  else LAUNCH(T, 64)
+#define LAUNCH(T, R, VEC)                                                                                          \
+  hipLaunchKernelGGL((linear_state_kernel<T, R, VEC>), grid, block, 0, stream, (const T*)r, (const T*)k,             \
+                     (const T*)v, r_stride, k_stride, v_stride, w_rows, w_head, a_rows, b_rows, state, state_stride, \
+                     q_start, state_slots, out, heads, dim, vdim, silu)
+#define PICK(T)                                              \
+  if (vec16 && dim == 32) LAUNCH(T, 8, true);                \
+  else if (vec16 && dim == 64) LAUNCH(T, 16, true);          \
+  else if (vec16 && dim == 128) LAUNCH(T, 32, true);         \
+  else if (vec16 && dim == 256) LAUNCH(T, 64, true);         \
+  else if (dim <= 16) LAUNCH(T, 4, false);                   \
+  else if (dim <= 32) LAUNCH(T, 8, false);                   \
+  else if (dim <= 64) LAUNCH(T, 16, false);                  \
+  else if (dim <= 128) LAUNCH(T, 32, false);                 \
+  else LAUNCH(T, 64, false)
   if (dtype == IX_F32) { PICK(float); }
   else if (dtype == IX_BF16) { PICK(bf16_t); }
   else IX_REQUIRE(false, "dtype must be float32 or bfloat16");
