@@ -35,6 +35,26 @@ __device__ __forceinline__ void ls_load8(const bf16_t* p, float (&o)[8]) {
   o[6] = __uint_as_float(a.w << 16); o[7] = __uint_as_float(a.w & 0xffff0000u);
 }
 
+// eight consecutive numbers as they come from memory, opened into floats when they are used
+template <typename T> struct ls_piece;
+template <> struct ls_piece<float> { float4 a, b; };
+template <> struct ls_piece<bf16_t> { uint4 a; };
+__device__ __forceinline__ void ls_ask8(const float* p, ls_piece<float>& o) {
+  o.a = *reinterpret_cast<const float4*>(p);
+  o.b = *reinterpret_cast<const float4*>(p + 4);
+}
+__device__ __forceinline__ void ls_ask8(const bf16_t* p, ls_piece<bf16_t>& o) { o.a = *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ void ls_open8(const ls_piece<float>& x, float (&o)[8]) {
+  o[0] = x.a.x; o[1] = x.a.y; o[2] = x.a.z; o[3] = x.a.w;
+  o[4] = x.b.x; o[5] = x.b.y; o[6] = x.b.z; o[7] = x.b.w;
+}
+__device__ __forceinline__ void ls_open8(const ls_piece<bf16_t>& x, float (&o)[8]) {
+  o[0] = __uint_as_float(x.a.x << 16); o[1] = __uint_as_float(x.a.x & 0xffff0000u);
+  o[2] = __uint_as_float(x.a.y << 16); o[3] = __uint_as_float(x.a.y & 0xffff0000u);
+  o[4] = __uint_as_float(x.a.z << 16); o[5] = __uint_as_float(x.a.z & 0xffff0000u);
+  o[6] = __uint_as_float(x.a.w << 16); o[7] = __uint_as_float(x.a.w & 0xffff0000u);
+}
+
 // R: rows of a column per lane (4 R >= dim).  VEC: dim = 4 R, R a multiple of 8 and everything on 16-byte boundaries,
 // so that a lane reads its part of the state and of every operand in 16-byte pieces.
 template <typename T, int R, bool VEC>
@@ -136,12 +156,13 @@ linear_state_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* _
 }
 
 // The same recurrence for requests that bring many rows (prompt portions).  The operands of a row are the same for
-// every column of a head, so a workgroup of four wavefronts shares them: it brings LS_CHUNK rows of r and k (and of
+// every column of a head, so a workgroup of four wavefronts shares them: it brings CH rows of r and k (and of
 // w, a, b) into LDS at a time, as float32 and through silu where asked, all loads of a chunk in flight at once and a
 // chunk ahead of the arithmetic.  SP lanes share a column (RPL = dim / SP rows each, in registers), so a workgroup
 // owns 256 / SP columns, and a row costs a lane five (or two) reads of RPL numbers from LDS, three sweeps over
-// them and two sums over SP lanes.  CORR: w, a, b come per row and channel; else the decay is one number per head.
-#define LS_CHUNK 16
+// them and two sums over SP lanes.  The rows are a chain, so what counts is how short a row is and how many
+// wavefronts there are: heads of 64 and 128 numbers take 32 lanes a column (1,024 wavefronts for 16 heads of 128
+// columns: one on every SIMD of the machine).  CORR: w, a, b come per row and channel; else the decay is one number per head.
 #define LS_THREADS 256
 
 template <int SP>
@@ -150,10 +171,30 @@ __device__ __forceinline__ float ls_sum_over(float x) {  // over the SP neighbou
   x += ix_dpp<IX_DPP_XOR2>(x);
   if constexpr (SP >= 8) x += ix_dpp<IX_DPP_HALF_MIRROR>(x);
   if constexpr (SP >= 16) x += ix_dpp<IX_DPP_MIRROR>(x);
+  if constexpr (SP >= 32) {
+    // rows of 16 lanes in pairs: the odd row takes the even row's total through DPP (row_bcast15: lane 15 of the
+    // row before, for rows 1 and 3), and the pair's total goes from its last lane to all of its lanes as a scalar
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
+    const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 31));
+    const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+    x = (threadIdx.x & 32) ? hi : lo;
+  }
   return x;
 }
 
-template <typename T, int SP, int RPL, bool CORR>
+// the same sum where only the last of the SP lanes needs it
+template <int SP>
+__device__ __forceinline__ float ls_sum_last(float x) {
+  x += ix_dpp<IX_DPP_XOR1>(x);
+  x += ix_dpp<IX_DPP_XOR2>(x);
+  if constexpr (SP >= 8) x += ix_dpp<IX_DPP_HALF_MIRROR>(x);
+  if constexpr (SP >= 16) x += ix_dpp<IX_DPP_MIRROR>(x);
+  if constexpr (SP >= 32)
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
+  return x;
+}
+
+template <typename T, int SP, int RPL, bool CORR, int CH>  // CH: rows per chunk
 __global__ void __launch_bounds__(LS_THREADS)
 linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, int64_t r_stride,
                           int64_t k_stride, int64_t v_stride, const float* __restrict__ w_rows,
@@ -164,14 +205,14 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
   constexpr int DIM = SP * RPL;
   constexpr int COLS = LS_THREADS / SP;                 // value columns of a workgroup
   constexpr int P8 = DIM / 8, P4 = DIM / 4;             // pieces of a row: of eight numbers (r, k), of four (w, a, b)
-  constexpr int RK_PIECES = LS_CHUNK * 2 * P8;
+  constexpr int RK_PIECES = CH * 2 * P8;
   constexpr int RK_PER = (RK_PIECES + LS_THREADS - 1) / LS_THREADS;
-  constexpr int WAB_PIECES = CORR ? LS_CHUNK * 3 * P4 : 0;
+  constexpr int WAB_PIECES = CORR ? CH * 3 * P4 : 0;
   constexpr int WAB_PER = CORR ? (WAB_PIECES + LS_THREADS - 1) / LS_THREADS : 1;
-  constexpr int V_PER = (LS_CHUNK * COLS + LS_THREADS - 1) / LS_THREADS;
-  __shared__ float4 rk_s[LS_CHUNK][2][P4];              // [row][k, r]
-  __shared__ float4 wab_s[CORR ? LS_CHUNK : 1][3][P4];  // [row][w, a, b]
-  __shared__ float v_s[LS_CHUNK][COLS];
+  constexpr int V_PER = (CH * COLS + LS_THREADS - 1) / LS_THREADS;
+  __shared__ float4 rk_s[CH][2][P4];              // [row][k, r]
+  __shared__ float4 wab_s[CORR ? CH : 1][3][P4];  // [row][w, a, b]
+  __shared__ float v_s[CH][COLS];
   const int tid = threadIdx.x;
   const int col0 = blockIdx.x * COLS;
   const int col = col0 + tid / SP, part = tid % SP;
@@ -183,24 +224,34 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
   const int cj = live ? col : vdim - 1;  // lanes past the last column repeat it and store nothing
   float* sp = state + static_cast<int64_t>(state_slots[seq]) * state_stride +
               (static_cast<int64_t>(head) * vdim + cj) * DIM + part * RPL;
-  float S[RPL];
+  // RPL numbers that lie side by side (RPL is 2 or a multiple of 4), to and from registers
+  auto take = [](const float* src, float (&dst)[RPL]) {
+    if constexpr (RPL == 2) {
+      const float2 x = *reinterpret_cast<const float2*>(src);
+      dst[0] = x.x; dst[1] = x.y;
+    } else {
 #pragma unroll
-  for (int i = 0; i < RPL; i += 4) {
-    const float4 x = *reinterpret_cast<const float4*>(sp + i);
-    S[i] = x.x; S[i + 1] = x.y; S[i + 2] = x.z; S[i + 3] = x.w;
-  }
+      for (int i = 0; i < RPL; i += 4) {
+        const float4 x = *reinterpret_cast<const float4*>(src + i);
+        dst[i] = x.x; dst[i + 1] = x.y; dst[i + 2] = x.z; dst[i + 3] = x.w;
+      }
+    }
+  };
+  float S[RPL];
+  take(sp, S);
   const float wh = CORR ? 1.0f : w_head[head];
   const int64_t chan = static_cast<int64_t>(heads) * DIM;  // channels of a row of w, a, b
 
-  float st_rk[RK_PER][8], st_v[V_PER];
+  ls_piece<T> st_rk[RK_PER];
+  float st_v[V_PER];
   float4 st_wab[WAB_PER];
-  auto ask = [&](int first) {  // rows first .. first + LS_CHUNK - 1 of the portion (rows past its end repeat the last)
+  auto ask = [&](int first) {  // rows first .. first + CH - 1 of the portion (rows past its end repeat the last)
 #pragma unroll
     for (int u = 0; u < RK_PER; ++u) {
       const int id = min(u * LS_THREADS + tid, RK_PIECES - 1);
       const int row = id / (2 * P8), which = (id / P8) & 1, pc = id % P8;
       const int64_t at = row0 + min(first + row, n - 1);
-      ls_load8((which ? r + at * r_stride : k + at * k_stride) + head * DIM + 8 * pc, st_rk[u]);
+      ls_ask8((which ? r + at * r_stride : k + at * k_stride) + head * DIM + 8 * pc, st_rk[u]);
     }
     if constexpr (CORR) {
 #pragma unroll
@@ -213,7 +264,7 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
     }
 #pragma unroll
     for (int u = 0; u < V_PER; ++u) {
-      const int id = min(u * LS_THREADS + tid, LS_CHUNK * COLS - 1);
+      const int id = min(u * LS_THREADS + tid, CH * COLS - 1);
       const int row = id / COLS, c = id % COLS;
       st_v[u] = ix_load(v + (row0 + min(first + row, n - 1)) * v_stride + head * vdim + min(col0 + c, vdim - 1));
     }
@@ -225,8 +276,11 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
       if (id < RK_PIECES) {
         const int row = id / (2 * P8), which = (id / P8) & 1, pc = id % P8;
         float x[8];
+        ls_open8(st_rk[u], x);
+        if (silu) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = silu ? ls_silu(st_rk[u][e]) : st_rk[u][e];
+          for (int e = 0; e < 8; ++e) x[e] = ls_silu(x[e]);
+        }
         rk_s[row][which][2 * pc] = float4{x[0], x[1], x[2], x[3]};
         rk_s[row][which][2 * pc + 1] = float4{x[4], x[5], x[6], x[7]};
       }
@@ -241,63 +295,53 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
 #pragma unroll
     for (int u = 0; u < V_PER; ++u) {
       const int id = u * LS_THREADS + tid;
-      if (id < LS_CHUNK * COLS) v_s[id / COLS][id % COLS] = silu ? ls_silu(st_v[u]) : st_v[u];
+      if (id < CH * COLS) v_s[id / COLS][id % COLS] = silu ? ls_silu(st_v[u]) : st_v[u];
     }
   };
-  auto fetch = [&](int row, float4 (&kk)[RPL / 4], float4 (&rr)[RPL / 4], float4 (&ww)[RPL / 4], float4 (&aa)[RPL / 4],
-                   float4 (&bb)[RPL / 4], float& vv) {
-#pragma unroll
-    for (int j = 0; j < RPL / 4; ++j) {
-      kk[j] = rk_s[row][0][part * (RPL / 4) + j];
-      rr[j] = rk_s[row][1][part * (RPL / 4) + j];
-      if constexpr (CORR) {
-        ww[j] = wab_s[row][0][part * (RPL / 4) + j];
-        aa[j] = wab_s[row][1][part * (RPL / 4) + j];
-        bb[j] = wab_s[row][2][part * (RPL / 4) + j];
-      }
+  auto fetch = [&](int row, float (&kk)[RPL], float (&rr)[RPL], float (&ww)[RPL], float (&aa)[RPL], float (&bb)[RPL],
+                   float& vv) {
+    take(reinterpret_cast<const float*>(&rk_s[row][0][0]) + part * RPL, kk);
+    take(reinterpret_cast<const float*>(&rk_s[row][1][0]) + part * RPL, rr);
+    if constexpr (CORR) {
+      take(reinterpret_cast<const float*>(&wab_s[row][0][0]) + part * RPL, ww);
+      take(reinterpret_cast<const float*>(&wab_s[row][1][0]) + part * RPL, aa);
+      take(reinterpret_cast<const float*>(&wab_s[row][2][0]) + part * RPL, bb);
     }
     vv = v_s[row][tid / SP];
   };
 
   ask(0);
-  for (int first = 0; first < n; first += LS_CHUNK) {
+  for (int first = 0; first < n; first += CH) {
     __syncthreads();  // the chunk before has been read
     put();
     __syncthreads();
-    if (first + LS_CHUNK < n) ask(first + LS_CHUNK);  // on their way while this chunk is worked
+    if (first + CH < n) ask(first + CH);  // on their way while this chunk is worked
     __builtin_amdgcn_sched_barrier(0);
-    const int rows = min(LS_CHUNK, n - first);
-    float4 kc[RPL / 4], rc[RPL / 4], wc[RPL / 4], ac[RPL / 4], bc[RPL / 4];
+    const int rows = min(CH, n - first);
+    float kc[RPL], rc[RPL], wc[RPL], ac[RPL], bc[RPL];
     float vc;
     fetch(0, kc, rc, wc, ac, bc, vc);
     for (int i = 0; i < rows; ++i) {
-      float4 kn[RPL / 4], rn[RPL / 4], wn[RPL / 4], an[RPL / 4], bn[RPL / 4];
+      float kn[RPL], rn[RPL], wn[RPL], an[RPL], bn[RPL];
       float vn;
-      fetch(min(i + 1, LS_CHUNK - 1), kn, rn, wn, an, bn, vn);
+      fetch(min(i + 1, CH - 1), kn, rn, wn, an, bn, vn);
       float read = 0.f;
       if constexpr (CORR) {
 #pragma unroll
-        for (int j = 0; j < RPL / 4; ++j)
-          read += bc[j].x * S[4 * j] + bc[j].y * S[4 * j + 1] + bc[j].z * S[4 * j + 2] + bc[j].w * S[4 * j + 3];
+        for (int j = 0; j < RPL; ++j) read += bc[j] * S[j];
         read = ls_sum_over<SP>(read);
       }
       float o = 0.f;
 #pragma unroll
-      for (int j = 0; j < RPL / 4; ++j) {
-        const float ke[4] = {kc[j].x, kc[j].y, kc[j].z, kc[j].w}, re[4] = {rc[j].x, rc[j].y, rc[j].z, rc[j].w};
-        const float we[4] = {wc[j].x, wc[j].y, wc[j].z, wc[j].w}, ae[4] = {ac[j].x, ac[j].y, ac[j].z, ac[j].w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float& s = S[4 * j + e];
-          if constexpr (CORR) s = we[e] * s - ae[e] * read + ke[e] * vc;
-          else s = wh * s + ke[e] * vc;
-          o += re[e] * s;
-        }
+      for (int j = 0; j < RPL; ++j) {
+        if constexpr (CORR) S[j] = wc[j] * S[j] - ac[j] * read + kc[j] * vc;
+        else S[j] = wh * S[j] + kc[j] * vc;
+        o += rc[j] * S[j];
       }
-      o = ls_sum_over<SP>(o);
-      if (live && part == 0) out[((row0 + first + i) * heads + head) * vdim + col] = o;
+      o = ls_sum_last<SP>(o);
+      if (live && part == SP - 1) out[((row0 + first + i) * heads + head) * vdim + col] = o;
 #pragma unroll
-      for (int j = 0; j < RPL / 4; ++j) {
+      for (int j = 0; j < RPL; ++j) {
         kc[j] = kn[j];
         rc[j] = rn[j];
         if constexpr (CORR) {
@@ -310,8 +354,12 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
     }
   }
   if (live) {
+    if constexpr (RPL == 2) {
+      *reinterpret_cast<float2*>(sp) = float2{S[0], S[1]};
+    } else {
 #pragma unroll
-    for (int i = 0; i < RPL; i += 4) *reinterpret_cast<float4*>(sp + i) = float4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+      for (int i = 0; i < RPL; i += 4) *reinterpret_cast<float4*>(sp + i) = float4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+    }
   }
 }
 
@@ -342,15 +390,15 @@ extern "C" int ix_linear_state(const void* r, const void* k, const void* v, int 
     if ((dtype == IX_F32 || dtype == IX_BF16) && (corr || none) && aligned && tokens >= 4 * static_cast<int64_t>(requests) &&
         (dim == 16 || dim == 32 || dim == 64 || dim == 128)) {
 #define CHUNKED(T, SP, RPL, CORR)                                                                                        \
-  hipLaunchKernelGGL((linear_state_chunk_kernel<T, SP, RPL, CORR>),                                                      \
+  hipLaunchKernelGGL((linear_state_chunk_kernel<T, SP, RPL, CORR, (CORR ? (SP * RPL >= 128 ? 16 : 32) : 64)>),                                                      \
                      dim3((vdim + LS_THREADS / SP - 1) / (LS_THREADS / SP), heads, requests), dim3(LS_THREADS), 0, stream, \
                      (const T*)r, (const T*)k, (const T*)v, r_stride, k_stride, v_stride, w_rows, w_head, a_rows, b_rows, \
                      state, state_stride, q_start, state_slots, out, heads, vdim, silu)
 #define BY_DIM(T, CORR)                            \
   if (dim == 16) CHUNKED(T, 4, 4, CORR);           \
   else if (dim == 32) CHUNKED(T, 8, 4, CORR);      \
-  else if (dim == 64) CHUNKED(T, 16, 4, CORR);     \
-  else CHUNKED(T, 16, 8, CORR)
+  else if (dim == 64) CHUNKED(T, 32, 2, CORR);     \
+  else CHUNKED(T, 32, 4, CORR)
       if (dtype == IX_F32) {
         if (corr) { BY_DIM(float, true); } else { BY_DIM(float, false); }
       } else {
