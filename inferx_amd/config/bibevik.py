@@ -101,6 +101,8 @@ def _mlp(raw: Any, where: str) -> Optional[BibevikMlp]:
     if raw is None:
         return None
     kind = _number(raw, "kind", where, str)
+    if kind not in MLP_KINDS:
+        raise ConfigError(f"config.json: {where}.kind {kind!r} is not known (known: " + ", ".join(MLP_KINDS) + ")")
     if kind == "dense":
         return BibevikMlp(kind, ff=_number(raw, "ff", where, int), limit=_number(raw, "limit", where, float))
     router, expert = raw.get("router"), raw.get("expert")
