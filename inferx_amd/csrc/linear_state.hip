@@ -163,7 +163,6 @@ linear_state_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* _
 // them and two sums over SP lanes.  The rows are a chain, so what counts is how short a row is and how many
 // wavefronts there are: heads of 64 and 128 numbers take 32 lanes a column (1,024 wavefronts for 16 heads of 128
 // columns: one on every SIMD of the machine).  CORR: w, a, b come per row and channel; else the decay is one number per head.
-#define LS_THREADS 256
 
 template <int SP>
 __device__ __forceinline__ float ls_sum_over(float x) {  // over the SP neighbouring lanes of a column
@@ -171,7 +170,13 @@ __device__ __forceinline__ float ls_sum_over(float x) {  // over the SP neighbou
   x += ix_dpp<IX_DPP_XOR2>(x);
   if constexpr (SP >= 8) x += ix_dpp<IX_DPP_HALF_MIRROR>(x);
   if constexpr (SP >= 16) x += ix_dpp<IX_DPP_MIRROR>(x);
-  if constexpr (SP >= 32) {
+  if constexpr (SP >= 64) {
+    // all four rows of 16 lanes: rows 1 and 3 take the row before, rows 2 and 3 the first pair's total (row_bcast31:
+    // lane 31, for rows 2 and 3); the last lane's total goes to all lanes as a scalar
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x143, 0xc, 0xf, false));
+    x = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+  } else if constexpr (SP >= 32) {
     // rows of 16 lanes in pairs: the odd row takes the even row's total through DPP (row_bcast15: lane 15 of the
     // row before, for rows 1 and 3), and the pair's total goes from its last lane to all of its lanes as a scalar
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
@@ -191,11 +196,13 @@ __device__ __forceinline__ float ls_sum_last(float x) {
   if constexpr (SP >= 16) x += ix_dpp<IX_DPP_MIRROR>(x);
   if constexpr (SP >= 32)
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
+  if constexpr (SP >= 64)
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x143, 0xc, 0xf, false));
   return x;
 }
 
-template <typename T, int SP, int RPL, bool CORR, int CH>  // CH: rows per chunk
-__global__ void __launch_bounds__(LS_THREADS)
+template <typename T, int SP, int RPL, bool CORR, int CH, int THREADS>  // CH: rows per chunk; THREADS per workgroup
+__global__ void __launch_bounds__(THREADS)
 linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, int64_t r_stride,
                           int64_t k_stride, int64_t v_stride, const float* __restrict__ w_rows,
                           const float* __restrict__ w_head, const float* __restrict__ a_rows,
@@ -203,13 +210,13 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
                           const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
                           float* __restrict__ out, int heads, int vdim, int silu) {
   constexpr int DIM = SP * RPL;
-  constexpr int COLS = LS_THREADS / SP;                 // value columns of a workgroup
+  constexpr int COLS = THREADS / SP;                 // value columns of a workgroup
   constexpr int P8 = DIM / 8, P4 = DIM / 4;             // pieces of a row: of eight numbers (r, k), of four (w, a, b)
   constexpr int RK_PIECES = CH * 2 * P8;
-  constexpr int RK_PER = (RK_PIECES + LS_THREADS - 1) / LS_THREADS;
+  constexpr int RK_PER = (RK_PIECES + THREADS - 1) / THREADS;
   constexpr int WAB_PIECES = CORR ? CH * 3 * P4 : 0;
-  constexpr int WAB_PER = CORR ? (WAB_PIECES + LS_THREADS - 1) / LS_THREADS : 1;
-  constexpr int V_PER = (CH * COLS + LS_THREADS - 1) / LS_THREADS;
+  constexpr int WAB_PER = CORR ? (WAB_PIECES + THREADS - 1) / THREADS : 1;
+  constexpr int V_PER = (CH * COLS + THREADS - 1) / THREADS;
   __shared__ float4 rk_s[CH][2][P4];              // [row][k, r]
   __shared__ float4 wab_s[CORR ? CH : 1][3][P4];  // [row][w, a, b]
   __shared__ float v_s[CH][COLS];
@@ -248,7 +255,7 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
   auto ask = [&](int first) {  // rows first .. first + CH - 1 of the portion (rows past its end repeat the last)
 #pragma unroll
     for (int u = 0; u < RK_PER; ++u) {
-      const int id = min(u * LS_THREADS + tid, RK_PIECES - 1);
+      const int id = min(u * THREADS + tid, RK_PIECES - 1);
       const int row = id / (2 * P8), which = (id / P8) & 1, pc = id % P8;
       const int64_t at = row0 + min(first + row, n - 1);
       ls_ask8((which ? r + at * r_stride : k + at * k_stride) + head * DIM + 8 * pc, st_rk[u]);
@@ -256,7 +263,7 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
     if constexpr (CORR) {
 #pragma unroll
       for (int u = 0; u < WAB_PER; ++u) {
-        const int id = min(u * LS_THREADS + tid, WAB_PIECES - 1);
+        const int id = min(u * THREADS + tid, WAB_PIECES - 1);
         const int row = id / (3 * P4), which = (id / P4) % 3, pc = id % P4;
         const float* src = which == 0 ? w_rows : (which == 1 ? a_rows : b_rows);
         st_wab[u] = *reinterpret_cast<const float4*>(src + (row0 + min(first + row, n - 1)) * chan + head * DIM + 4 * pc);
@@ -264,7 +271,7 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
     }
 #pragma unroll
     for (int u = 0; u < V_PER; ++u) {
-      const int id = min(u * LS_THREADS + tid, CH * COLS - 1);
+      const int id = min(u * THREADS + tid, CH * COLS - 1);
       const int row = id / COLS, c = id % COLS;
       st_v[u] = ix_load(v + (row0 + min(first + row, n - 1)) * v_stride + head * vdim + min(col0 + c, vdim - 1));
     }
@@ -272,7 +279,7 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
   auto put = [&]() {
 #pragma unroll
     for (int u = 0; u < RK_PER; ++u) {
-      const int id = u * LS_THREADS + tid;
+      const int id = u * THREADS + tid;
       if (id < RK_PIECES) {
         const int row = id / (2 * P8), which = (id / P8) & 1, pc = id % P8;
         float x[8];
@@ -288,13 +295,13 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
     if constexpr (CORR) {
 #pragma unroll
       for (int u = 0; u < WAB_PER; ++u) {
-        const int id = u * LS_THREADS + tid;
+        const int id = u * THREADS + tid;
         if (id < WAB_PIECES) wab_s[id / (3 * P4)][(id / P4) % 3][id % P4] = st_wab[u];
       }
     }
 #pragma unroll
     for (int u = 0; u < V_PER; ++u) {
-      const int id = u * LS_THREADS + tid;
+      const int id = u * THREADS + tid;
       if (id < CH * COLS) v_s[id / COLS][id % COLS] = silu ? ls_silu(st_v[u]) : st_v[u];
     }
   };
@@ -321,7 +328,9 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
     float kc[RPL], rc[RPL], wc[RPL], ac[RPL], bc[RPL];
     float vc;
     fetch(0, kc, rc, wc, ac, bc, vc);
-    for (int i = 0; i < rows; ++i) {
+    float* op = out + ((row0 + first) * heads + head) * vdim + (live ? col : 0);
+    const int64_t o_step = static_cast<int64_t>(heads) * vdim;
+    auto row_step = [&](int i) {
       float kn[RPL], rn[RPL], wn[RPL], an[RPL], bn[RPL];
       float vn;
       fetch(min(i + 1, CH - 1), kn, rn, wn, an, bn, vn);
@@ -339,7 +348,7 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
         o += rc[j] * S[j];
       }
       o = ls_sum_last<SP>(o);
-      if (live && part == SP - 1) out[((row0 + first + i) * heads + head) * vdim + col] = o;
+      if (live && part == SP - 1) op[i * o_step] = o;
 #pragma unroll
       for (int j = 0; j < RPL; ++j) {
         kc[j] = kn[j];
@@ -351,6 +360,14 @@ linear_state_chunk_kernel(const T* __restrict__ r, const T* __restrict__ k, cons
         }
       }
       vc = vn;
+    };
+    // a whole chunk with the rows' places in LDS known when the code is built (eight rows a turn of the loop: the
+    // copies from one row's operands to the next become names, the addresses constants); the last chunk row by row
+    if (rows == CH) {
+#pragma unroll 8
+      for (int i = 0; i < CH; ++i) row_step(i);
+    } else {
+      for (int i = 0; i < rows; ++i) row_step(i);
     }
   }
   if (live) {
@@ -389,16 +406,16 @@ extern "C" int ix_linear_state(const void* r, const void* k, const void* v, int 
     vec16 = aligned;
     if ((dtype == IX_F32 || dtype == IX_BF16) && (corr || none) && aligned && tokens >= 4 * static_cast<int64_t>(requests) &&
         (dim == 16 || dim == 32 || dim == 64 || dim == 128)) {
-#define CHUNKED(T, SP, RPL, CORR)                                                                                        \
-  hipLaunchKernelGGL((linear_state_chunk_kernel<T, SP, RPL, CORR, (CORR ? (SP * RPL >= 128 ? 16 : 32) : 64)>),                                                      \
-                     dim3((vdim + LS_THREADS / SP - 1) / (LS_THREADS / SP), heads, requests), dim3(LS_THREADS), 0, stream, \
+#define CHUNKED(T, SP, RPL, CORR, THREADS)                                                                               \
+  hipLaunchKernelGGL((linear_state_chunk_kernel<T, SP, RPL, CORR, (CORR ? (SP * RPL >= 128 ? 16 : 32) : 64), THREADS>),  \
+                     dim3((vdim + THREADS / SP - 1) / (THREADS / SP), heads, requests), dim3(THREADS), 0, stream,        \
                      (const T*)r, (const T*)k, (const T*)v, r_stride, k_stride, v_stride, w_rows, w_head, a_rows, b_rows, \
                      state, state_stride, q_start, state_slots, out, heads, vdim, silu)
-#define BY_DIM(T, CORR)                            \
-  if (dim == 16) CHUNKED(T, 4, 4, CORR);           \
-  else if (dim == 32) CHUNKED(T, 8, 4, CORR);      \
-  else if (dim == 64) CHUNKED(T, 32, 2, CORR);     \
-  else CHUNKED(T, 32, 4, CORR)
+#define BY_DIM(T, CORR)                                 \
+  if (dim == 16) CHUNKED(T, 4, 4, CORR, 256);           \
+  else if (dim == 32) CHUNKED(T, 8, 4, CORR, 256);      \
+  else if (dim == 64) CHUNKED(T, 32, 2, CORR, 256);     \
+  else CHUNKED(T, 64, 2, CORR, 512)
       if (dtype == IX_F32) {
         if (corr) { BY_DIM(float, true); } else { BY_DIM(float, false); }
       } else {
