@@ -415,7 +415,8 @@ extern "C" int ix_linear_state(const void* r, const void* k, const void* v, int 
   if (dim == 16) CHUNKED(T, 4, 4, CORR, 256);           \
   else if (dim == 32) CHUNKED(T, 8, 4, CORR, 256);      \
   else if (dim == 64) CHUNKED(T, 32, 2, CORR, 256);     \
-  else CHUNKED(T, 64, 2, CORR, 512)
+  else if (static_cast<int64_t>(heads) * vdim >= 4096) CHUNKED(T, 32, 4, CORR, 256); \
+  else CHUNKED(T, 64, 2, CORR, 512) /* few columns: a wavefront each, two wavefronts a SIMD at 2,048 of them */
       if (dtype == IX_F32) {
         if (corr) { BY_DIM(float, true); } else { BY_DIM(float, false); }
       } else {

@@ -47,7 +47,7 @@ def step_rows(lengths, slots):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("corrected", [True, False])
-@pytest.mark.parametrize("H,D,V", [(2, 16, 24), (3, 20, 12), (1, 32, 40), (2, 64, 64), (2, 128, 80), (1, 192, 16)])
+@pytest.mark.parametrize("H,D,V", [(2, 16, 24), (3, 20, 12), (1, 32, 40), (2, 64, 64), (2, 128, 80), (1, 192, 16), (32, 128, 128)])
 def test_recurrence_over_steps_and_slots(H, D, V, corrected, dtype):
     """Three requests in slots that are not in order: a step of unequal portions (several chunks, a chunk's edge, one
     row), then steps of one row each, then a portion of two rows: outputs and the state that is left against the
@@ -71,7 +71,7 @@ def test_recurrence_over_steps_and_slots(H, D, V, corrected, dtype):
             a = (u * torch.sigmoid(rnd((T, H * D), 10 * n + 6))).contiguous()
             w_head = None
         else:
-            w_head = torch.tensor([0.97, 0.6, 1.0][:H], dtype=torch.float32)
+            w_head = torch.tensor(([0.97, 0.6, 1.0] * H)[:H], dtype=torch.float32)
         out = torch.empty(T, H, V, dtype=torch.float32, device=DEV)
         ops.linear_state(r.to(DEV), k.to(DEV), v.to(DEV), state, step_rows(lengths, slots), out, H, D, V,
                          w_rows=w.to(DEV) if corrected else None, w_head=None if corrected else w_head.to(DEV),
