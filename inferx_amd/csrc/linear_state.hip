@@ -156,13 +156,15 @@ linear_state_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* _
 }
 
 // The same recurrence for requests that bring many rows (prompt portions).  The operands of a row are the same for
-// every column of a head, so a workgroup of four wavefronts shares them: it brings CH rows of r and k (and of
+// every column of a head, so a workgroup (THREADS / 64 wavefronts) shares them: it brings CH rows of r and k (and of
 // w, a, b) into LDS at a time, as float32 and through silu where asked, all loads of a chunk in flight at once and a
 // chunk ahead of the arithmetic.  SP lanes share a column (RPL = dim / SP rows each, in registers), so a workgroup
-// owns 256 / SP columns, and a row costs a lane five (or two) reads of RPL numbers from LDS, three sweeps over
-// them and two sums over SP lanes.  The rows are a chain, so what counts is how short a row is and how many
-// wavefronts there are: heads of 64 and 128 numbers take 32 lanes a column (1,024 wavefronts for 16 heads of 128
-// columns: one on every SIMD of the machine).  CORR: w, a, b come per row and channel; else the decay is one number per head.
+// owns THREADS / SP columns, and a row costs a lane five (or two) reads of RPL numbers from LDS, three sweeps over
+// them and two sums over SP lanes (DPP all the way: within a row of 16 lanes, then row_bcast15 and row_bcast31
+// across rows, the total taken from the last lane).  The rows are a chain, so what counts is how few instructions
+// a row is and how many wavefronts there are: heads of 64 numbers take 32 lanes a column, heads of 128 a whole
+// wavefront while that makes at most two wavefronts a SIMD (2,048 for 16 heads of 128 columns), else 32 lanes.
+// CORR: w, a, b come per row and channel; else the decay is one number per head.
 
 template <int SP>
 __device__ __forceinline__ float ls_sum_over(float x) {  // over the SP neighbouring lanes of a column
