@@ -50,11 +50,13 @@ def step_rows(lengths, slots):
 @pytest.mark.parametrize("H,D,V", [(2, 16, 24), (3, 20, 12), (1, 32, 40), (2, 64, 64), (2, 128, 80), (1, 192, 16), (32, 128, 128)])
 def test_recurrence_over_steps_and_slots(H, D, V, corrected, dtype):
     """Three requests in slots that are not in order: a step of unequal portions (several chunks, a chunk's edge, one
-    row), then steps of one row each, then a portion of two rows: outputs and the state that is left against the
-    float64 loop over the rows."""
+    row), then steps of one row each, then a portion of two rows, then portions around the longest chunk's length:
+    outputs and the state that is left against the float64 loop over the rows."""
     from inferx_amd import ops
     silu = not corrected
     steps = [(33, 16, 1), (1, 1, 1), (1, 1, 1), (2, 17, 5)]
+    if H <= 3:  # portions longer than the longest chunk: two whole chunks and two rows, a whole chunk, a chunk and a row
+        steps.append((130, 64, 65))
     slots = [4, 0, 2]
     state = torch.zeros(6, H * D * V + 8, dtype=torch.float32, device=DEV)
     state[1] = float("nan")  # a slot that nobody owns
