@@ -10,9 +10,11 @@ from . import dezudra  # registers Dezudra
 from .dezudra import DezudraConfig
 from . import bibevik  # registers Bibevik
 from .bibevik import BibevikConfig
+from . import gosuvik  # registers Gosuvik
+from .gosuvik import GosuvikConfig
 
 __all__ = [
     "ConfigError", "config_class_for", "config_from_dict", "config_from_directory", "config_from_json",
     "known_architectures", "register_architecture", "LayerSpec", "ModelSpec", "PartSpec", "ScheduleEntry", "linear_head", "token_embedding",
-    "Qwen2MoeConfig", "PelalixConfig", "DezudraConfig", "BibevikConfig",
+    "Qwen2MoeConfig", "PelalixConfig", "DezudraConfig", "BibevikConfig", "GosuvikConfig",
 ]

@@ -9,6 +9,11 @@
 // window rule :346-354).  Query head h reads kv head h / (heads / kv_heads).
 // Key j of a request lives in page table[j / page_size] at offset j % page_size;
 // keys are stored [page][kv_head][offset][d], values [page][kv_head][d][offset].
+// Values may be of another size than keys (`value_dim`).  `sink` (one float per head, or null): the softmax's
+// denominator also holds exp(sink[head]), which has no key and no value, is not scaled and counts once: the running
+// maximum starts there with a sum of one.  `turn_back` (float32 (cos, sin) [T, value_dim / 2], or null): the result
+// of every head is rotated by minus the query's angles, pair (i, i + value_dim / 2), before it is rounded (for
+// values that were cached rotated by their own positions).
 #include "common.h"
 
 #define ATTN_PLAIN_THREADS 256
@@ -18,7 +23,8 @@ __global__ void __launch_bounds__(ATTN_PLAIN_THREADS)
 attn_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                   const int32_t* __restrict__ block_table, const int32_t* __restrict__ seq_of_token,
                   const int32_t* __restrict__ positions, T* __restrict__ out, int heads, int kv_heads, int head_dim,
-                  int page_size, int max_blocks, float scale, int window) {
+                  int value_dim, int page_size, int max_blocks, float scale, int window,
+                  const float* __restrict__ sink, const float2* __restrict__ turn_back) {
   __shared__ float qs[256];
   __shared__ float sc[ATTN_PLAIN_THREADS];
   __shared__ int32_t pg[ATTN_PLAIN_THREADS];
@@ -36,7 +42,7 @@ attn_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const 
   if (tid < head_dim) qs[tid] = ix_load(q + (t * heads + head) * head_dim + tid);
   __syncthreads();
 
-  float m = -INFINITY, l = 0.f, acc = 0.f;
+  float m = sink ? sink[head] : -INFINITY, l = sink ? 1.f : 0.f, acc = 0.f;
   for (int base = start; base <= pos; base += ATTN_PLAIN_THREADS) {
     const int j = base + tid;
     const bool live = j <= pos;
@@ -57,39 +63,53 @@ attn_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const 
     const float alpha = expf(m - m_new);           // exp(-inf) = 0 on the first chunk
     l = l * alpha + chunk_sum;
     m = m_new;
-    if (tid < head_dim) {
+    if (tid < value_dim) {
       acc *= alpha;
       const int n = min(ATTN_PLAIN_THREADS, pos + 1 - base);
       for (int jj = 0; jj < n; ++jj) {
         const int key = base + jj;
         const T* vr =
-            v_cache + ((static_cast<int64_t>(pg[jj]) * kv_heads + g) * head_dim + tid) * page_size + key % page_size;
+            v_cache + ((static_cast<int64_t>(pg[jj]) * kv_heads + g) * value_dim + tid) * page_size + key % page_size;
         acc += sc[jj] * ix_load(vr);
       }
     }
     __syncthreads();
   }
-  if (tid < head_dim) ix_store(out + (t * heads + head) * head_dim + tid, acc / l);
+  float o = acc / l;
+  if (turn_back) {  // (the loop's last barrier has passed: `sc` is free)
+    if (tid < value_dim) sc[tid] = o;
+    __syncthreads();
+    const int half = value_dim / 2;
+    if (tid < 2 * half) {
+      const bool low = tid < half;
+      const float2 c = turn_back[t * half + (low ? tid : tid - half)];
+      const float other = sc[low ? tid + half : tid - half];
+      o = low ? o * c.x + other * c.y : o * c.x - other * c.y;
+    }
+  }
+  if (tid < value_dim) ix_store(out + (t * heads + head) * value_dim + tid, o);
 }
 
 extern "C" int ix_attention_plain(const void* q, const void* k_cache, const void* v_cache, int dtype,
                                   const int32_t* block_table, const int32_t* seq_of_token, const int32_t* positions,
-                                  void* out, int64_t tokens, int heads, int kv_heads, int head_dim, int page_size,
-                                  int max_blocks, float scale, int window, hipStream_t stream) {
+                                  void* out, int64_t tokens, int heads, int kv_heads, int head_dim, int value_dim,
+                                  int page_size, int max_blocks, float scale, int window, const float* sink,
+                                  const float* turn_back, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && page_size > 0 && max_blocks > 0, "sizes must be positive");
   IX_REQUIRE(heads % kv_heads == 0, "heads must be a multiple of kv_heads");
   IX_REQUIRE(head_dim > 0 && head_dim <= 256, "head_dim must be between 1 and 256");
+  IX_REQUIRE(value_dim > 0 && value_dim <= 256, "value_dim must be between 1 and 256");
   IX_REQUIRE(window >= 0, "window must not be negative");
   if (tokens == 0) return 0;
   dim3 grid(tokens, heads), block(ATTN_PLAIN_THREADS);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(attn_plain_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_cache,
                        (const float*)v_cache, block_table, seq_of_token, positions, (float*)out, heads, kv_heads,
-                       head_dim, page_size, max_blocks, scale, window);
+                       head_dim, value_dim, page_size, max_blocks, scale, window, sink, (const float2*)turn_back);
   else if (dtype == IX_BF16)
     hipLaunchKernelGGL(attn_plain_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache,
                        (const bf16_t*)v_cache, block_table, seq_of_token, positions, (bf16_t*)out, heads, kv_heads,
-                       head_dim, page_size, max_blocks, scale, window);
+                       head_dim, value_dim, page_size, max_blocks, scale, window, sink, (const float2*)turn_back);
   else
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_attention_plain");

@@ -7,6 +7,10 @@
 // size come from two small projections a, b (float32):  g = exp(-exp(A_log) softplus(a + dt_bias)),  beta =
 // sigmoid(b).  Everything but the loads of q, k, v is float32.
 //
+// A decay per key channel (`ach` given): g is a vector over the rows of S, g_i = exp(-exp(A_log) softplus(a_i +
+// dt_bias_i)) with a float32 [T, heads * dim] and dt_bias [heads * dim], S <- diag(g) S; `ab` then holds the step
+// size's logits alone, float32 [T, heads].
+//
 // The columns of S are independent recurrences (column j only ever meets v[j]), so the work is spread over
 // (request, head, block of 16 value columns): one wavefront each, four lanes per column that own every fourth row
 // of it (RPL rows a lane, in registers; VEC: a quarter of the rows each, side by side, where that quarter is a
@@ -37,10 +41,11 @@ __device__ __forceinline__ void delta_load8(const bf16_t* p, float (&out)[8]) {
   out[6] = __uint_as_float(a.w << 16); out[7] = __uint_as_float(a.w & 0xffff0000u);
 }
 
-template <typename T, int RPL, bool VEC>
+template <typename T, int RPL, bool VEC, bool CH>
 __global__ void __launch_bounds__(64)
 delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int64_t q_stride,
-                  int64_t k_stride, int64_t v_stride, const float* __restrict__ ab, const float* __restrict__ a_log,
+                  int64_t k_stride, int64_t v_stride, const float* __restrict__ ab, const float* __restrict__ ach,
+                  const float* __restrict__ a_log,
                   const float* __restrict__ dt_bias, float* __restrict__ state, int64_t state_stride,
                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
                   float* __restrict__ out, int heads, int kv_heads, int dim, int vdim) {
@@ -79,13 +84,45 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
       S[r] = i < dim ? sp[static_cast<int64_t>(cj) * dim + i] : 0.f;
     }
   }
-  const float rate = expf(a_log[head]), bias = dt_bias[head];
+  const float rate = expf(a_log[head]), bias = CH ? 0.f : dt_bias[head];
   const float q_scale = 1.0f / sqrtf(static_cast<float>(dim));
+  float biasr[CH ? RPL : 1];  // a decay per key channel: the bias of each of this lane's rows
+  if constexpr (CH) {
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+      const int i = row_of(r);
+      biasr[r] = i < dim ? dt_bias[head * dim + i] : 0.f;
+    }
+  }
 
   float kc[RPL], qc[RPL], vc, ac, bc;  // the present row's operands
-  auto fetch = [&](int64_t row, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& aa, float& bb) {
+  float gc[CH ? RPL : 1];               // (and the decay's logits of this lane's rows)
+  auto fetch = [&](int64_t row, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& aa, float& bb,
+                   float (&gg)[CH ? RPL : 1]) {
     const T* qr = q + row * q_stride + kv * dim;
     const T* kr = k + row * k_stride + kv * dim;
+    if constexpr (CH) {
+      const float* ar = ach + (row * heads + head) * dim;
+      if constexpr (VEC) {
+#pragma unroll
+        for (int r = 0; r < RPL; r += 4) {
+          if (r < quarter) {
+            const delta_f32x4 x = *reinterpret_cast<const delta_f32x4*>(ar + part * quarter + r);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) gg[r + e] = x[e];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) gg[r + e] = 0.f;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+          const int i = r * DELTA_SPLIT + part;
+          gg[r] = i < dim ? ar[i] : 0.f;
+        }
+      }
+    }
     if constexpr (VEC) {
 #pragma unroll
       for (int r = 0; r < RPL; r += 8) {
@@ -112,13 +149,18 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
       }
     }
     vv = ix_load(v + row * v_stride + head * vdim + cj);
-    aa = ab[row * 2 * heads + head];
-    bb = ab[row * 2 * heads + heads + head];
+    if constexpr (CH) {
+      aa = 0.f;
+      bb = ab[row * heads + head];
+    } else {
+      aa = ab[row * 2 * heads + head];
+      bb = ab[row * 2 * heads + heads + head];
+    }
   };
-  fetch(row0, kc, qc, vc, ac, bc);
+  fetch(row0, kc, qc, vc, ac, bc, gc);
   for (int i = 0; i < n; ++i) {
-    float kn[RPL], qn[RPL], vn, an, bn;
-    fetch(row0 + min(i + 1, n - 1), kn, qn, vn, an, bn);  // the next row's, on their way while this one is worked
+    float kn[RPL], qn[RPL], vn, an, bn, gn[CH ? RPL : 1];
+    fetch(row0 + min(i + 1, n - 1), kn, qn, vn, an, bn, gn);  // the next row's, on their way while this one is worked
     float kk = 0.f, qq = 0.f;
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
@@ -137,7 +179,12 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
     float dot = 0.f;
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
-      S[r] *= g;
+      if constexpr (CH) {
+        const float xr = gc[r] + biasr[r];
+        S[r] *= expf(-rate * (xr > 20.f ? xr : log1pf(expf(xr))));
+      } else {
+        S[r] *= g;
+      }
       dot += S[r] * (kc[r] * k_inv);
     }
     dot += ix_dpp<IX_DPP_XOR1>(dot);
@@ -156,6 +203,7 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
     for (int r = 0; r < RPL; ++r) {
       kc[r] = kn[r];
       qc[r] = qn[r];
+      if constexpr (CH) gc[r] = gn[r];
     }
     vc = vn;
     ac = an;
@@ -201,10 +249,10 @@ __device__ __forceinline__ float delta_sum_over(float x) {  // over the SP neigh
   return x;
 }
 
-template <int SP, int RPL>
+template <int SP, int RPL, bool CH>
 __global__ void __launch_bounds__(64)
 delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64_t q_stride, int64_t k_stride,
-                        int64_t v_stride, const float* ab, const float* __restrict__ a_log,
+                        int64_t v_stride, const float* ab, const float* ach, const float* __restrict__ a_log,
                         const float* __restrict__ dt_bias, float* __restrict__ state, int64_t state_stride,
                         const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
                         float* __restrict__ out, int heads, int kv_heads, int vdim) {
@@ -216,6 +264,9 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
   __shared__ delta_f32x4 qk_s[DELTA_CHUNK][2][DIM / 4];  // [row][k, q]: unit vectors (q times dim^(-1/2))
   __shared__ float v_s[DELTA_CHUNK][COLS];
   __shared__ float gb_s[DELTA_CHUNK][2];             // decay, step size
+  constexpr int G4 = DIM / 4;                        // 16-byte pieces of a row of decays (8, 16 or 32: divides 64)
+  constexpr int G_PER_LANE = CH ? DELTA_CHUNK * G4 / 64 : 1;
+  __shared__ delta_f32x4 g_s[CH ? DELTA_CHUNK : 1][CH ? G4 : 1];  // a decay per key channel: [row][channel]
   const int lane = threadIdx.x;
   const int col0 = blockIdx.x * COLS;
   const int col = col0 + lane / SP, part = lane % SP;
@@ -231,12 +282,24 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
   float S[RPL];
 #pragma unroll
   for (int r = 0; r < RPL; ++r) S[r] = sp[static_cast<int64_t>(cj) * DIM + part * RPL + r];
-  const float rate = expf(a_log[head]), bias = dt_bias[head];
+  const float rate = expf(a_log[head]), bias = CH ? 0.f : dt_bias[head];
   const float q_scale = 1.0f / sqrtf(static_cast<float>(DIM));
+  // (piece u * 64 + lane of a chunk's decays is piece lane % G4 of a row whatever u: the bias is the lane's own)
+  delta_f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (CH) bias4 = *reinterpret_cast<const delta_f32x4*>(dt_bias + head * DIM + 4 * (lane % G4));
 
   delta_u32x4 st_qk[PER_LANE];
+  delta_f32x4 st_g[G_PER_LANE];
   float st_v[V_PER_LANE], st_ab;
-  auto ask = [&](int first) {  // rows first .. first + DELTA_CHUNK - 1 of the portion (rows past its end repeat the last)
+  auto ask = [&](int first) {
+    if constexpr (CH) {
+#pragma unroll
+      for (int u = 0; u < G_PER_LANE; ++u) {
+        const int id = u * 64 + lane;
+        const int64_t row = row0 + min(first + id / G4, n - 1);
+        st_g[u] = *reinterpret_cast<const delta_f32x4*>(ach + (row * heads + head) * DIM + 4 * (id % G4));
+      }
+    }  // rows first .. first + DELTA_CHUNK - 1 of the portion (rows past its end repeat the last)
 #pragma unroll
     for (int u = 0; u < PER_LANE; ++u) {
       const int id = u * 64 + lane;  // piece number within the chunk: [row][k, q][piece]
@@ -253,7 +316,8 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
     }
     {
       const int r = lane / 2, which = lane & 1;
-      st_ab = ab[(row0 + min(first + r, n - 1)) * 2 * heads + which * heads + head];
+      if constexpr (CH) st_ab = ab[(row0 + min(first + r, n - 1)) * heads + head];
+      else st_ab = ab[(row0 + min(first + r, n - 1)) * 2 * heads + which * heads + head];
     }
   };
   auto put = [&]() {
@@ -282,12 +346,34 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
     }
     if (lane & 1) {
       gb_s[lane / 2][1] = 1.0f / (1.0f + expf(-st_ab));
-    } else {
+    } else if constexpr (!CH) {
       const float x = st_ab + bias;
       gb_s[lane / 2][0] = expf(-rate * (x > 20.f ? x : log1pf(expf(x))));
     }
+    if constexpr (CH) {
+#pragma unroll
+      for (int u = 0; u < G_PER_LANE; ++u) {
+        const int id = u * 64 + lane;
+        delta_f32x4 g;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float x = st_g[u][e] + bias4[e];
+          g[e] = expf(-rate * (x > 20.f ? x : log1pf(expf(x))));
+        }
+        g_s[id / G4][id % G4] = g;
+      }
+    }
   };
-  auto fetch = [&](int r, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& gg, float& bb) {
+  auto fetch = [&](int r, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& gg, float& bb,
+                   float (&gr)[CH ? RPL : 1]) {
+    if constexpr (CH) {
+#pragma unroll
+      for (int j = 0; j < RPL / 4; ++j) {
+        const delta_f32x4 a = g_s[r][part * (RPL / 4) + j];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gr[4 * j + e] = a[e];
+      }
+    }
 #pragma unroll
     for (int j = 0; j < RPL / 4; ++j) {
       const delta_f32x4 a = qk_s[r][0][part * (RPL / 4) + j], b = qk_s[r][1][part * (RPL / 4) + j];
@@ -298,7 +384,7 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
       }
     }
     vv = v_s[r][lane / SP];
-    gg = gb_s[r][0];
+    gg = CH ? 1.0f : gb_s[r][0];
     bb = gb_s[r][1];
   };
 
@@ -310,14 +396,17 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
     if (first + DELTA_CHUNK < n) ask(first + DELTA_CHUNK);  // on their way while this chunk is worked
     __builtin_amdgcn_sched_barrier(0);
     const int rows = min(DELTA_CHUNK, n - first);
-    float kc[RPL], qc[RPL], vc, gc, bc;
-    fetch(0, kc, qc, vc, gc, bc);
+    float kc[RPL], qc[RPL], vc, gc, bc, grc[CH ? RPL : 1];
+    fetch(0, kc, qc, vc, gc, bc, grc);
     for (int i = 0; i < rows; ++i) {
-      float kn[RPL], qn[RPL], vn, gn, bn;
-      fetch(min(i + 1, DELTA_CHUNK - 1), kn, qn, vn, gn, bn);
+      float kn[RPL], qn[RPL], vn, gn, bn, grn[CH ? RPL : 1];
+      fetch(min(i + 1, DELTA_CHUNK - 1), kn, qn, vn, gn, bn, grn);
       float dot = 0.f;
 #pragma unroll
-      for (int r = 0; r < RPL; ++r) dot += S[r] * kc[r];
+      for (int r = 0; r < RPL; ++r) {
+        if constexpr (CH) S[r] *= grc[r];
+        dot += S[r] * kc[r];
+      }
       dot = delta_sum_over<SP>(dot);
       const float u = bc * (vc - gc * dot);
       float o = 0.f;
@@ -332,6 +421,7 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
       for (int r = 0; r < RPL; ++r) {
         kc[r] = kn[r];
         qc[r] = qn[r];
+        if constexpr (CH) grc[r] = grn[r];
       }
       vc = vn;
       gc = gn;
@@ -345,10 +435,11 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
 }
 
 // q, k [T, kv_heads * dim] and v [T, heads * vdim] of the run's type with their row strides; ab float32 [T, 2 heads]
-// (a then b); a_log, dt_bias float32 [heads]; state: slot s at state + s * state_stride, [heads, vdim, dim] (a column's rows side by side);
+// (a then b); a_log, dt_bias float32 [heads]; or, with a decay per key channel, ach float32 [T, heads * dim], ab
+// float32 [T, heads] (b alone) and dt_bias float32 [heads * dim]; state: slot s at state + s * state_stride, [heads, vdim, dim] (a column's rows side by side);
 // out float32 [T, heads, vdim].
 extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dtype, int64_t q_stride,
-                             int64_t k_stride, int64_t v_stride, const float* ab, const float* a_log,
+                             int64_t k_stride, int64_t v_stride, const float* ab, const float* ach, const float* a_log,
                              const float* dt_bias, float* state, int64_t state_stride, const int32_t* q_start,
                              const int32_t* state_slots, float* out, int64_t tokens, int requests, int heads,
                              int kv_heads, int dim, int vdim, hipStream_t stream) {
@@ -365,11 +456,17 @@ extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dt
   const int elt = 2;
   const bool vec = dtype == IX_BF16 && dim % (8 * DELTA_SPLIT) == 0 && (q_stride * elt) % 16 == 0 && (k_stride * elt) % 16 == 0 &&
                    state_stride % 4 == 0 &&
-                   ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(state)) & 15) == 0;
-#define LAUNCH(TT, RPL, VEC)                                                                                            \
-  hipLaunchKernelGGL((delta_rule_kernel<TT, RPL, VEC>), grid, block, 0, stream, (const TT*)q, (const TT*)k, (const TT*)v, \
-                     q_stride, k_stride, v_stride, ab, a_log, dt_bias, state, state_stride, q_start, state_slots, out,    \
+                   ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(state) |
+                     reinterpret_cast<uintptr_t>(ach) | reinterpret_cast<uintptr_t>(dt_bias)) & 15) == 0;
+#define LAUNCH_CH(TT, RPL, VEC, CH)                                                                                         \
+  hipLaunchKernelGGL((delta_rule_kernel<TT, RPL, VEC, CH>), grid, block, 0, stream, (const TT*)q, (const TT*)k, (const TT*)v, \
+                     q_stride, k_stride, v_stride, ab, ach, a_log, dt_bias, state, state_stride, q_start, state_slots, out,   \
                      heads, kv_heads, dim, vdim)
+#define LAUNCH(TT, RPL, VEC)                \
+  do {                                      \
+    if (ach) LAUNCH_CH(TT, RPL, VEC, true); \
+    else LAUNCH_CH(TT, RPL, VEC, false);    \
+  } while (0)
 #define PICK(TT, VEC)                      \
   if (rpl <= 8) LAUNCH(TT, 8, VEC);        \
   else if (rpl <= 16) LAUNCH(TT, 16, VEC); \
@@ -377,20 +474,27 @@ extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dt
   else LAUNCH(TT, 64, VEC);
   // steps that bring a request many rows: chunks through LDS (heads of 32, 64 or 128 numbers)
   if (vec && tokens >= 4 * static_cast<int64_t>(requests) && (dim == 32 || dim == 64 || dim == 128)) {
-#define CHUNKED(SP, RPL)                                                                                                  \
-  hipLaunchKernelGGL((delta_rule_chunk_kernel<SP, RPL>), dim3((vdim + 64 / SP - 1) / (64 / SP), heads, requests), block, 0, \
-                     stream, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, q_stride, k_stride, v_stride, ab, a_log, \
-                     dt_bias, state, state_stride, q_start, state_slots, out, heads, kv_heads, vdim)
+#define CHUNKED_CH(SP, RPL, CH)                                                                                               \
+  hipLaunchKernelGGL((delta_rule_chunk_kernel<SP, RPL, CH>), dim3((vdim + 64 / SP - 1) / (64 / SP), heads, requests), block, \
+                     0, stream, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, q_stride, k_stride, v_stride, ab, ach, \
+                     a_log, dt_bias, state, state_stride, q_start, state_slots, out, heads, kv_heads, vdim)
+#define CHUNKED(SP, RPL)                \
+  do {                                  \
+    if (ach) CHUNKED_CH(SP, RPL, true); \
+    else CHUNKED_CH(SP, RPL, false);    \
+  } while (0)
     if (dim == 32) CHUNKED(4, 8);
     else if (dim == 64) CHUNKED(16, 4);
     else CHUNKED(16, 8);
 #undef CHUNKED
+#undef CHUNKED_CH
     return ix_check_launch("ix_delta_rule");
   }
   // (the 16-byte form is built for bfloat16, the type whose runs are timed)
   if (dtype == IX_F32) { PICK(float, false) } else if (vec) { PICK(bf16_t, true) } else { PICK(bf16_t, false) }
 #undef PICK
 #undef LAUNCH
+#undef LAUNCH_CH
   return ix_check_launch("ix_delta_rule");
 }
 

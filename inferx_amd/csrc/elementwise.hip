@@ -46,12 +46,14 @@ extern "C" int ix_embed(void* h, const void* table, int table_dtype, const int32
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, const void* __restrict__ w,
                                    int w_dtype, TO* __restrict__ out, const int32_t* __restrict__ rows,
-                                   int64_t width, float eps) {
+                                   int64_t row_width, int64_t width, float eps) {
+  // (`width` is what one norm runs over: the row, or one of its gridDim.y equal runs, each with its own sum)
   __shared__ float red[16];
   const int64_t r = blockIdx.x;
   const int64_t row = rows ? rows[r] : r;
-  float* hr = h + row * width;
-  const TD* dr = delta ? delta + row * width : nullptr;
+  const int64_t first = blockIdx.y * width;
+  float* hr = h + row * row_width + first;
+  const TD* dr = delta ? delta + row * row_width + first : nullptr;
   const bool write_back = (rows == nullptr) && (dr != nullptr);
   float sumsq = 0.f;
   for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
@@ -62,23 +64,25 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   }
   sumsq = ix_block_sum(sumsq, red);
   const float inv = 1.0f / sqrtf(sumsq / static_cast<float>(width) + eps);
-  TO* outr = out + r * width;
+  TO* outr = out + r * row_width + first;
   for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
     float v = hr[i];
     if (dr && !write_back) v += ix_load(dr + i);
-    ix_store(outr + i, v * inv * ix_load_rt(w, w_dtype, i));
+    ix_store(outr + i, v * inv * ix_load_rt(w, w_dtype, first + i));
   }
 }
 
 // bfloat16 delta and output with a width that is a multiple of 4: four columns per thread
 __global__ void add_rmsnorm_vec4_kernel(float* __restrict__ h, const uint16_t* __restrict__ delta,
                                         const void* __restrict__ w, int w_dtype, uint16_t* __restrict__ out,
-                                        const int32_t* __restrict__ rows, int64_t width, float eps) {
+                                        const int32_t* __restrict__ rows, int64_t row_width, int64_t width,
+                                        float eps) {
   __shared__ float red[16];
   const int64_t r = blockIdx.x;
   const int64_t row = rows ? rows[r] : r;
-  float* hr = h + row * width;
-  const uint16_t* dr = delta ? delta + row * width : nullptr;
+  const int64_t first = blockIdx.y * width;
+  float* hr = h + row * row_width + first;
+  const uint16_t* dr = delta ? delta + row * row_width + first : nullptr;
   const bool write_back = (rows == nullptr) && (dr != nullptr);
   auto value = [&](int64_t c) {
     float4 v = *reinterpret_cast<const float4*>(hr + c);
@@ -101,33 +105,36 @@ __global__ void add_rmsnorm_vec4_kernel(float* __restrict__ h, const uint16_t* _
   }
   sumsq = ix_block_sum(sumsq, red);
   const float inv = 1.0f / sqrtf(sumsq / static_cast<float>(width) + eps);
-  uint16_t* outr = out + r * width;
+  uint16_t* outr = out + r * row_width + first;
   for (int64_t c = 4 * threadIdx.x; c < width; c += 4 * blockDim.x) {
     const float4 v = value(c);  // h is still as it was: it is written here, after its last reading
     if (write_back) *reinterpret_cast<float4*>(hr + c) = v;
     uint2 o;
-    o.x = ix_f32_to_bf16(v.x * inv * ix_load_rt(w, w_dtype, c)) |
-          static_cast<uint32_t>(ix_f32_to_bf16(v.y * inv * ix_load_rt(w, w_dtype, c + 1))) << 16;
-    o.y = ix_f32_to_bf16(v.z * inv * ix_load_rt(w, w_dtype, c + 2)) |
-          static_cast<uint32_t>(ix_f32_to_bf16(v.w * inv * ix_load_rt(w, w_dtype, c + 3))) << 16;
+    o.x = ix_f32_to_bf16(v.x * inv * ix_load_rt(w, w_dtype, first + c)) |
+          static_cast<uint32_t>(ix_f32_to_bf16(v.y * inv * ix_load_rt(w, w_dtype, first + c + 1))) << 16;
+    o.y = ix_f32_to_bf16(v.z * inv * ix_load_rt(w, w_dtype, first + c + 2)) |
+          static_cast<uint32_t>(ix_f32_to_bf16(v.w * inv * ix_load_rt(w, w_dtype, first + c + 3))) << 16;
     *reinterpret_cast<uint2*>(outr + c) = o;
   }
 }
 
 extern "C" int ix_add_rmsnorm(void* h, const void* delta, int delta_dtype, const void* w, int w_dtype, void* out,
-                              int out_dtype, const int32_t* rows, int64_t n_out_rows, int64_t width, float eps,
-                              hipStream_t stream) {
-  IX_REQUIRE(width > 0 && n_out_rows >= 0, "sizes must be positive");
+                              int out_dtype, const int32_t* rows, int64_t n_out_rows, int64_t row_width, int groups,
+                              float eps, hipStream_t stream) {
+  // `groups`: the row is cut into that many equal runs, each normalised by its own root mean square
+  IX_REQUIRE(row_width > 0 && n_out_rows >= 0, "sizes must be positive");
+  IX_REQUIRE(groups > 0 && groups <= 65535 && row_width % groups == 0, "the groups must divide the width");
   IX_REQUIRE(w_dtype == IX_F32 || w_dtype == IX_BF16, "weight dtype must be float32 or bfloat16");
   if (n_out_rows == 0) return 0;
-  dim3 grid(n_out_rows), block(width >= 4096 ? 1024 : (width >= 1024 ? 512 : 256));
+  const int64_t width = row_width / groups;
+  dim3 grid(n_out_rows, groups), block(width >= 4096 ? 1024 : (width >= 1024 ? 512 : 256));
 #define LAUNCH(TD, TO)                                                                                          \
   hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), grid, block, 0, stream, (float*)h, (const TD*)delta, w, w_dtype, \
-                     (TO*)out, rows, width, eps)
+                     (TO*)out, rows, row_width, width, eps)
   if (out_dtype == IX_BF16 && (delta == nullptr || delta_dtype == IX_BF16) && width % 4 == 0 &&
       ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(delta) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
     hipLaunchKernelGGL(add_rmsnorm_vec4_kernel, grid, dim3(width >= 4096 ? 1024 : (width >= 2048 ? 512 : 256)), 0, stream,
-                       (float*)h, (const uint16_t*)delta, w, w_dtype, (uint16_t*)out, rows, width, eps);
+                       (float*)h, (const uint16_t*)delta, w, w_dtype, (uint16_t*)out, rows, row_width, width, eps);
     return ix_check_launch("ix_add_rmsnorm");
   }
   if (delta_dtype == IX_F32 && out_dtype == IX_F32) LAUNCH(float, float);
@@ -228,7 +235,7 @@ extern "C" int ix_add_bias(void* y, int dtype, const void* bias, int bias_dtype,
 // (reference: RopeKernel, layers.cu:80-115, which recomputes the angle per head
 // with fast intrinsics; here it is computed once per step with sincosf)
 __global__ void rope_table_kernel(float2* __restrict__ cs, const int32_t* __restrict__ positions,
-                                  const float* __restrict__ inv_freq, int64_t tokens, int half) {
+                                  const float* __restrict__ inv_freq, int64_t tokens, int half, float gain) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= tokens * half) return;
   const int64_t t = i / half;
@@ -236,16 +243,17 @@ __global__ void rope_table_kernel(float2* __restrict__ cs, const int32_t* __rest
   const float a = static_cast<float>(positions[t]) * inv_freq[j];
   float s, c;
   sincosf(a, &s, &c);
-  cs[i] = make_float2(c, s);
+  cs[i] = make_float2(c * gain, s * gain);
 }
 
+// `gain`: what cosine and sine are multiplied by (1 for a plain rotation; stretched encodings lengthen the vectors)
 extern "C" int ix_rope_table(void* cs, const int32_t* positions, const float* inv_freq, int64_t tokens, int half,
-                             hipStream_t stream) {
+                             float gain, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && half > 0, "sizes must be positive");
   if (tokens == 0) return 0;
   const int64_t n = tokens * half;
   hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, (float2*)cs, positions, inv_freq,
-                     tokens, half);
+                     tokens, half, gain);
   return ix_check_launch("ix_rope_table");
 }
 
@@ -617,4 +625,103 @@ extern "C" int ix_add_branches(float* h, const void* a, const void* b, int dtype
   else
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_add_branches");
+}
+
+
+// ---------------------------------------------------------------------------
+// The PolyNorm activation, a workgroup per row:
+//   out = a N(z) + b N(z^2) + c N(z^3) + e,   N(v) = v / sqrt(mean(v^2) + eps)   (powers element by element)
+// The three sums of squares (of z, z^2, z^3) and the blend are float32; coef holds a, b, c, e.
+template <typename T>
+__global__ void __launch_bounds__(256)
+polynorm_kernel(const T* __restrict__ z, const void* __restrict__ coef, int c_dtype, T* __restrict__ out,
+                int64_t width, float eps) {
+  __shared__ float red[16];
+  const T* zr = z + static_cast<int64_t>(blockIdx.x) * width;
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = ix_load(zr + i), v2 = v * v;
+    s1 += v2;
+    s2 += v2 * v2;
+    s3 += v2 * v2 * v2;
+  }
+  s1 = ix_block_sum(s1, red);
+  s2 = ix_block_sum(s2, red);
+  s3 = ix_block_sum(s3, red);
+  const float n = static_cast<float>(width);
+  const float f1 = ix_load_rt(coef, c_dtype, 0) / sqrtf(s1 / n + eps), f2 = ix_load_rt(coef, c_dtype, 1) / sqrtf(s2 / n + eps),
+              f3 = ix_load_rt(coef, c_dtype, 2) / sqrtf(s3 / n + eps), shift = ix_load_rt(coef, c_dtype, 3);
+  T* outr = out + static_cast<int64_t>(blockIdx.x) * width;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = ix_load(zr + i);
+    ix_store(outr + i, v * (f1 + v * (f2 + v * f3)) + shift);
+  }
+}
+
+extern "C" int ix_polynorm(const void* z, const void* coef, int c_dtype, void* out, int dtype, int64_t tokens,
+                           int64_t width, float eps, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  IX_REQUIRE(c_dtype == IX_F32 || c_dtype == IX_BF16, "the coefficients must be float32 or bfloat16");
+  if (tokens == 0) return 0;
+  dim3 grid(static_cast<unsigned>(tokens)), block(width >= 4096 ? 1024 : 256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(polynorm_kernel<float>, grid, block, 0, stream, (const float*)z, coef, c_dtype, (float*)out, width, eps);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(polynorm_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)z, coef, c_dtype, (bf16_t*)out, width, eps);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_polynorm");
+}
+
+// ---------------------------------------------------------------------------
+// out[i] = fa * a[i] + fb * b[i] in float32 (two branches' results with a constant gain each, on their way to the
+// residual stream); b may be null.
+template <typename T>
+__global__ void weighted_sum_kernel(const T* __restrict__ a, float fa, const T* __restrict__ b, float fb,
+                                    float* __restrict__ out, int64_t n) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    out[i] = b ? fa * ix_load(a + i) + fb * ix_load(b + i) : fa * ix_load(a + i);
+}
+
+extern "C" int ix_weighted_sum(const void* a, float fa, const void* b, float fb, int dtype, float* out, int64_t n,
+                               hipStream_t stream) {
+  IX_REQUIRE(n >= 0, "sizes must be positive");
+  if (n == 0) return 0;
+  dim3 grid(static_cast<unsigned>(std::min<int64_t>((n + 255) / 256, 65536))), block(256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(weighted_sum_kernel<float>, grid, block, 0, stream, (const float*)a, fa, (const float*)b, fb, out, n);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(weighted_sum_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)a, fa, (const bf16_t*)b, fb, out, n);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_weighted_sum");
+}
+
+// ---------------------------------------------------------------------------
+// y[t, c] *= sigmoid(gate[t * gate_stride + c]) in place (a gate on a mixer's result before its last product).
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ y, const T* __restrict__ gate, int64_t gate_stride, int64_t tokens,
+                                    int64_t width) {
+  const int64_t n = tokens * width;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = i / width, c = i - t * width;
+    ix_store(y + i, ix_load(y + i) / (1.0f + expf(-ix_load(gate + t * gate_stride + c))));
+  }
+}
+
+extern "C" int ix_sigmoid_gate(void* y, const void* gate, int64_t gate_stride, int dtype, int64_t tokens, int64_t width,
+                               hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0 && gate_stride >= width, "sizes must be positive");
+  if (tokens == 0) return 0;
+  const int64_t n = tokens * width;
+  dim3 grid(static_cast<unsigned>(std::min<int64_t>((n + 255) / 256, 65536))), block(256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, block, 0, stream, (float*)y, (const float*)gate, gate_stride, tokens, width);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, (const bf16_t*)gate, gate_stride, tokens, width);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_sigmoid_gate");
 }

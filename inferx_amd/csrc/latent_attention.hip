@@ -15,13 +15,14 @@
 //   q        rows of heads x q_dim numbers, q_stride apart; the last rot_dim of each head are the rotated part
 //   dkv      [T, >= rank + rot_dim] rows (may be strided)
 //   cos_sin  float32 [T, pairs, 2]: element 2i of a rotated part is paired with 2i + 1, i < pairs; the rest passes
+//            (`halves`: element i is paired with i + pairs instead, the first 2 * pairs numbers of the part)
 //   cache    [pages * page_size, rank + rot_dim]; slots[t] is the token's row
 template <typename T>
 __global__ void __launch_bounds__(256)
 latent_prepare_kernel(T* __restrict__ q, int64_t q_stride, const T* __restrict__ dkv, int64_t dkv_stride,
                       const void* __restrict__ norm_w, int nw_dtype, float eps, const float* __restrict__ cos_sin,
                       int pairs, const int32_t* __restrict__ slots, T* __restrict__ cache, int heads, int q_dim,
-                      int rot_dim, int rank) {
+                      int rot_dim, int rank, int halves) {
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
   const int tid = threadIdx.x;
@@ -29,10 +30,11 @@ latent_prepare_kernel(T* __restrict__ q, int64_t q_stride, const T* __restrict__
   // the queries' rotated parts
   for (int i = tid; i < heads * pairs; i += blockDim.x) {
     const int h = i / pairs, p = i - h * pairs;
-    T* at = q + t * q_stride + h * q_dim + (q_dim - rot_dim) + 2 * p;
-    const float u = ix_load(at), v = ix_load(at + 1), c = cs[2 * p], s = cs[2 * p + 1];
+    T* at = q + t * q_stride + h * q_dim + (q_dim - rot_dim) + (halves ? p : 2 * p);
+    T* with = at + (halves ? pairs : 1);
+    const float u = ix_load(at), v = ix_load(with), c = cs[2 * p], s = cs[2 * p + 1];
     ix_store(at, u * c - v * s);
-    ix_store(at + 1, v * c + u * s);
+    ix_store(with, v * c + u * s);
   }
   const T* row = dkv + t * dkv_stride;
   T* dst = slots ? cache + static_cast<int64_t>(slots[t]) * (rank + rot_dim) : nullptr;
@@ -46,6 +48,19 @@ latent_prepare_kernel(T* __restrict__ q, int64_t q_stride, const T* __restrict__
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(rank) + eps);
   for (int i = tid; i < rank; i += blockDim.x)
     ix_store(dst + i, ix_load(row + i) * inv * ix_load_rt(norm_w, nw_dtype, i));
+  if (halves) {
+    for (int i = tid; i < rot_dim; i += blockDim.x) {
+      const float x = ix_load(row + rank + i);
+      if (i < 2 * pairs) {
+        const int p = i < pairs ? i : i - pairs;
+        const float other = ix_load(row + rank + (i < pairs ? i + pairs : i - pairs)), c = cs[2 * p], s = cs[2 * p + 1];
+        ix_store(dst + rank + i, i < pairs ? x * c - other * s : x * c + other * s);
+      } else {
+        ix_store(dst + rank + i, x);
+      }
+    }
+    return;
+  }
   for (int p = tid; p < rot_dim / 2 + (rot_dim & 1); p += blockDim.x) {
     const int i = 2 * p;
     const float u = ix_load(row + rank + i);
@@ -62,7 +77,7 @@ latent_prepare_kernel(T* __restrict__ q, int64_t q_stride, const T* __restrict__
 
 extern "C" int ix_latent_prepare(void* q, int64_t q_stride, const void* dkv, int64_t dkv_stride, int dtype, const void* norm_w,
                                  int nw_dtype, float eps, const float* cos_sin, int pairs, const int32_t* slots,
-                                 void* cache, int64_t tokens, int heads, int q_dim, int rot_dim, int rank,
+                                 void* cache, int64_t tokens, int heads, int q_dim, int rot_dim, int rank, int halves,
                                  hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && heads > 0 && rank > 0 && rot_dim >= 0 && q_dim >= rot_dim, "sizes must be positive");
   IX_REQUIRE(pairs >= 0 && 2 * pairs <= rot_dim && (pairs == 0 || cos_sin != nullptr),
@@ -71,11 +86,11 @@ extern "C" int ix_latent_prepare(void* q, int64_t q_stride, const void* dkv, int
   dim3 grid(static_cast<unsigned>(tokens)), block(256);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(latent_prepare_kernel<float>, grid, block, 0, stream, (float*)q, q_stride, (const float*)dkv, dkv_stride,
-                       norm_w, nw_dtype, eps, cos_sin, pairs, slots, (float*)cache, heads, q_dim, rot_dim, rank);
+                       norm_w, nw_dtype, eps, cos_sin, pairs, slots, (float*)cache, heads, q_dim, rot_dim, rank, halves);
   else if (dtype == IX_BF16)
     hipLaunchKernelGGL(latent_prepare_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)q, q_stride, (const bf16_t*)dkv,
                        dkv_stride, norm_w, nw_dtype, eps, cos_sin, pairs, slots, (bf16_t*)cache, heads, q_dim, rot_dim,
-                       rank);
+                       rank, halves);
   else
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_latent_prepare");
@@ -97,7 +112,7 @@ latent_attn_plain_kernel(const T* __restrict__ ql, int64_t ql_t, int64_t ql_h, c
                          int64_t qr_h, const T* __restrict__ cache, const int32_t* __restrict__ block_table,
                          const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                          T* __restrict__ out, int64_t out_t, int64_t out_h, int rank, int rot_dim, int page_size,
-                         int max_blocks, float scale) {
+                         int max_blocks, float scale, int window) {
   __shared__ float qs[LAT_MAX_WIDTH];
   __shared__ float sc[LAT_THREADS];
   __shared__ int64_t at[LAT_THREADS];
@@ -112,7 +127,9 @@ latent_attn_plain_kernel(const T* __restrict__ ql, int64_t ql_t, int64_t ql_h, c
     qs[i] = i < rank ? ix_load(ql + t * ql_t + head * ql_h + i) : ix_load(qr + t * qr_t + head * qr_h + (i - rank));
   __syncthreads();
   float m = -INFINITY, l = 0.f, acc[LAT_ACC] = {0.f, 0.f, 0.f, 0.f};
-  for (int base = 0; base <= pos; base += LAT_THREADS) {
+  // with a window W a query reads the keys pos + 1 - W .. pos only (pages before them may be gone)
+  const int start = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  for (int base = start; base <= pos; base += LAT_THREADS) {
     const int j = base + tid;
     const bool live = j <= pos;
     float s = -INFINITY;
@@ -155,9 +172,9 @@ extern "C" int ix_latent_attention_plain(const void* ql, int64_t ql_t, int64_t q
                                          int64_t qr_h, const void* cache, int dtype, const int32_t* block_table,
                                          const int32_t* seq_of_token, const int32_t* positions, void* out,
                                          int64_t out_t, int64_t out_h, int64_t tokens, int heads, int rank,
-                                         int rot_dim, int page_size, int max_blocks, float scale,
+                                         int rot_dim, int page_size, int max_blocks, float scale, int window,
                                          hipStream_t stream) {
-  IX_REQUIRE(tokens >= 0 && heads > 0 && rank > 0 && rot_dim >= 0 && page_size > 0 && max_blocks > 0,
+  IX_REQUIRE(tokens >= 0 && heads > 0 && rank > 0 && rot_dim >= 0 && page_size > 0 && max_blocks > 0 && window >= 0,
              "sizes must be positive");
   IX_REQUIRE(rank <= LAT_ACC * LAT_THREADS && rank + rot_dim <= LAT_MAX_WIDTH,
              "the latent holds at most 1024 numbers, with the rotated part at most 1088");
@@ -167,11 +184,11 @@ extern "C" int ix_latent_attention_plain(const void* ql, int64_t ql_t, int64_t q
   if (dtype == IX_F32)
     hipLaunchKernelGGL(latent_attn_plain_kernel<float>, grid, block, 0, stream, (const float*)ql, ql_t, ql_h,
                        (const float*)qr, qr_t, qr_h, (const float*)cache, block_table, seq_of_token, positions,
-                       (float*)out, out_t, out_h, rank, rot_dim, page_size, max_blocks, scale);
+                       (float*)out, out_t, out_h, rank, rot_dim, page_size, max_blocks, scale, window);
   else if (dtype == IX_BF16)
     hipLaunchKernelGGL(latent_attn_plain_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)ql, ql_t, ql_h,
                        (const bf16_t*)qr, qr_t, qr_h, (const bf16_t*)cache, block_table, seq_of_token, positions,
-                       (bf16_t*)out, out_t, out_h, rank, rot_dim, page_size, max_blocks, scale);
+                       (bf16_t*)out, out_t, out_h, rank, rot_dim, page_size, max_blocks, scale, window);
   else
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_latent_attention_plain");
@@ -211,7 +228,8 @@ latent_attn_mfma_kernel(const __bf16* __restrict__ ql, int64_t ql_t, int64_t ql_
                         const int32_t* __restrict__ block_table, const int32_t* __restrict__ seq_of_token,
                         const int32_t* __restrict__ positions, __bf16* __restrict__ out, int64_t out_t, int64_t out_h,
                         float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits, int tokens, int heads,
-                        int rank, int rot_dim, int page_size, int max_blocks, float scale_log2, int n_tiles) {
+                        int rank, int rot_dim, int page_size, int max_blocks, float scale_log2, int n_tiles,
+                        int window) {
   extern __shared__ __attribute__((aligned(16))) unsigned char latm_lds[];
   constexpr int NP = (4 * NW + 7) / 8;  // 16-byte pieces of a round's rows that a thread moves
   const int width = rank + rot_dim;
@@ -268,20 +286,25 @@ latent_attn_mfma_kernel(const __bf16* __restrict__ ql, int64_t ql_t, int64_t ql_
     int end = seg + 1;
     if constexpr (!DEC)
       while (end < r1 && seq_of_token[end] == seq) ++end;
-    int k_begin = 0, k_end = positions[end - 1] + 1;  // a request's rows come in the order of their positions
+    int k_end = positions[end - 1] + 1;  // a request's rows come in the order of their positions
+    // with a window W the first of these rows reads from key k_lo on, and no row reads an earlier one (whose page
+    // may be gone); rounds start at multiples of their length
+    const int k_lo = window > 0 ? max(positions[seg] + 1 - window, 0) : 0;
+    int k_begin = k_lo & ~(LATM_KEYS - 1);
     if constexpr (DEC) {
-      const int per = ((k_end + n_splits - 1) / n_splits + LATM_KEYS - 1) & ~(LATM_KEYS - 1);
-      k_begin = static_cast<int>(blockIdx.z) * per;
+      const int per = ((k_end - k_begin + n_splits - 1) / n_splits + LATM_KEYS - 1) & ~(LATM_KEYS - 1);
+      k_begin += static_cast<int>(blockIdx.z) * per;
       k_end = min(k_end, k_begin + per);
     }
     const int my_pos = (col_ok && row >= seg && row < end) ? positions[row] : -1;
+    const int my_lo = window > 0 ? my_pos - window : -1;  // the last key that this column does not read
     const int32_t* table = block_table + static_cast<int64_t>(seq) * max_blocks;
 
     uint4 st[NP];
     const int my_key = tid >> 3, my_sub = tid & 7;  // a thread moves pieces my_sub, my_sub + 8, .. of one key's row
     auto ask = [&](int k0) {
       const int j = k0 + my_key;
-      const bool there = j < k_end;
+      const bool there = j < k_end && j >= k_lo;
       const int64_t at = there ? (static_cast<int64_t>(table[j / page_size]) * page_size + j % page_size) * width : 0;
 #pragma unroll
       for (int u = 0; u < NP; ++u) {
@@ -343,8 +366,8 @@ latent_attn_mfma_kernel(const __bf16* __restrict__ ql, int64_t ql_t, int64_t ql_
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int j = k0 + 8 * g + i;
-          p[i] = (j <= my_pos && j < k_end) ? s0[i] * scale_log2 : -INFINITY;
-          p[4 + i] = (j + 4 <= my_pos && j + 4 < k_end) ? s1[i] * scale_log2 : -INFINITY;
+          p[i] = (j <= my_pos && j > my_lo && j < k_end) ? s0[i] * scale_log2 : -INFINITY;
+          p[4 + i] = (j + 4 <= my_pos && j + 4 > my_lo && j + 4 < k_end) ? s1[i] * scale_log2 : -INFINITY;
           mx = fmaxf(mx, fmaxf(p[i], p[4 + i]));
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16));
@@ -410,9 +433,9 @@ extern "C" int ix_latent_attention_mfma(const void* ql, int64_t ql_t, int64_t ql
                                         const int32_t* seq_of_token, const int32_t* positions, void* out,
                                         int64_t out_t, int64_t out_h, float* part_o, float* part_ml, int n_splits,
                                         int64_t tokens, int heads, int rank, int rot_dim, int page_size,
-                                        int max_blocks, float scale, int decode, hipStream_t stream) {
-  IX_REQUIRE(tokens >= 0 && tokens < (1 << 30) && heads > 0 && rank > 0 && rot_dim >= 0 && page_size > 0 && max_blocks > 0,
-             "sizes must be positive");
+                                        int max_blocks, float scale, int decode, int window, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && tokens < (1 << 30) && heads > 0 && rank > 0 && rot_dim >= 0 && page_size > 0 && max_blocks > 0 &&
+                 window >= 0, "sizes must be positive");
   const int width = rank + rot_dim;
   IX_REQUIRE(width % 32 == 0 && rank % 16 == 0 && width <= 576 && rank <= 512,
              "rank + rot_dim must be a multiple of 32 up to 576, rank a multiple of 16 up to 512");
@@ -446,7 +469,7 @@ extern "C" int ix_latent_attention_mfma(const void* ql, int64_t ql_t, int64_t ql
     hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, (const __bf16*)ql, ql_t, ql_h, (const __bf16*)qr, qr_t,     \
                        qr_h, (const __bf16*)cache, block_table, seq_of_token, positions, (__bf16*)out, out_t, out_h,     \
                        part_o, part_ml, n_splits, static_cast<int>(tokens), heads, rank, rot_dim, page_size, max_blocks, \
-                       scale_log2, n_tiles);                                                                            \
+                       scale_log2, n_tiles, window);                                                                    \
   } while (0)
 #define BY_SIZE(DEC)                                        \
   if (width <= 128 && rank <= 128) LAUNCH(4, 8, DEC);       \

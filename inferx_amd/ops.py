@@ -95,10 +95,12 @@ def embed(h: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float 
 
 
 def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, out: torch.Tensor, eps: float,
-                rows: Optional[torch.Tensor] = None) -> None:
+                rows: Optional[torch.Tensor] = None, groups: int = 1) -> None:
     """out = rmsnorm(h + delta) * weight; h += delta in place when `rows` is None.
-    With `rows`, out[r] is computed from row rows[r] and h is not changed."""
+    With `rows`, out[r] is computed from row rows[r] and h is not changed.  `groups`: the width is cut into that
+    many equal runs, each divided by its own root mean square."""
     H = h.shape[1]
+    _need(groups >= 1 and H % groups == 0, "the groups must divide the width")
     _need(h.dtype == torch.float32, "the residual stream is float32")
     _need(weight.numel() == H and out.shape[1] == H, "width mismatch")
     n_out = out.shape[0]
@@ -109,7 +111,7 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     if delta is not None:
         _need(delta.shape == h.shape, "delta must have the shape of h")
     _call("ix_add_rmsnorm", _ptr(h), _ptr(delta), _i32(_dt(delta) if delta is not None else F32), _ptr(weight),
-          _i32(_dt(weight)), _ptr(out), _i32(_dt(out)), _ptr(rows), _i64(n_out), _i64(H), _f32(eps), _stream())
+          _i32(_dt(weight)), _ptr(out), _i32(_dt(out)), _ptr(rows), _i64(n_out), _i64(H), _i32(groups), _f32(eps), _stream())
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
@@ -126,13 +128,37 @@ def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
           _stream())
 
 
-def rope_table(cos_sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:
-    """cos_sin[t, j] = (cos, sin)(positions[t] * inv_freq[j]); float32 [T, half, 2]."""
+def rope_table(cos_sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, gain: float = 1.0) -> None:
+    """cos_sin[t, j] = (cos, sin)(positions[t] * inv_freq[j]) * gain; float32 [T, half, 2]."""
     T, half, two = cos_sin.shape
     _need(two == 2 and cos_sin.dtype == torch.float32 and inv_freq.dtype == torch.float32, "float32 tables needed")
     _need(inv_freq.numel() == half, "inv_freq length differs")
     _is_i32(positions, T)
-    _call("ix_rope_table", _ptr(cos_sin), _ptr(positions), _ptr(inv_freq), _i64(T), _i32(half), _stream())
+    _call("ix_rope_table", _ptr(cos_sin), _ptr(positions), _ptr(inv_freq), _i64(T), _i32(half), _f32(gain), _stream())
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, out: torch.Tensor, eps: float) -> None:
+    """out = a N(z) + b N(z^2) + c N(z^3) + e row by row, N(v) = v / sqrt(mean(v^2) + eps), coef = (a, b, c, e)."""
+    _need(z.dim() == 2 and z.is_contiguous() and out.shape == z.shape and out.dtype == z.dtype and out.is_contiguous(),
+          "z and out must be dense rows of one type")
+    _need(coef.numel() == 4 and coef.is_contiguous(), "four coefficients")
+    _call("ix_polynorm", _ptr(z), _ptr(coef), _i32(_dt(coef)), _ptr(out), _i32(_dt(z)), _i64(z.shape[0]), _i64(z.shape[1]),
+          _f32(eps), _stream())
+
+
+def weighted_sum(a: torch.Tensor, fa: float, b: Optional[torch.Tensor], fb: float, out: torch.Tensor) -> None:
+    """out = fa * a + fb * b, float32 (b may be None)."""
+    _need(a.is_contiguous() and out.dtype == torch.float32 and out.shape == a.shape and out.is_contiguous(), "dense operands")
+    _need(b is None or (b.shape == a.shape and b.dtype == a.dtype and b.is_contiguous()), "b must be like a")
+    _call("ix_weighted_sum", _ptr(a), _f32(fa), _ptr(b), _f32(fb), _i32(_dt(a)), _ptr(out), _i64(a.numel()), _stream())
+
+
+def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> None:
+    """y[t, c] *= sigmoid(gate[t, c]) in place; gate's rows may be strided."""
+    _need(y.dim() == 2 and y.is_contiguous() and gate.shape == y.shape and gate.dtype == y.dtype and gate.stride(1) == 1
+          and gate.is_cuda, "y dense, gate rows of y's type and width")
+    _call("ix_sigmoid_gate", _ptr(y), gate.data_ptr(), _i64(gate.stride(0)), _i32(_dt(y)), _i64(y.shape[0]), _i64(y.shape[1]),
+          _stream())
 
 
 def qkv_rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
@@ -208,19 +234,76 @@ def _check_caches(q, k_cache, v_cache):
 
 def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                     seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float,
-                    window: int) -> None:
-    """Paged attention, one workgroup per (token, head).  q, out [T, heads, d]."""
+                    window: int, sink: Optional[torch.Tensor] = None, turn_back: Optional[torch.Tensor] = None) -> None:
+    """Paged attention, one workgroup per (token, head).  q [T, heads, d], out [T, heads, value size] (the value
+    cache's).  `sink` float32 [heads]: exp(sink) joins every softmax's denominator, with no key and no value.
+    `turn_back` float32 [T, value size / 2, 2]: every head's result is rotated by minus these angles (halves paired)."""
     T, heads, d = q.shape
-    _need(out.shape == q.shape and out.dtype == q.dtype, "out mismatch")
-    _check_caches(q, k_cache, v_cache)
+    vd = v_cache.shape[2]
+    _need(out.shape == (T, heads, vd) and out.dtype == q.dtype, "out mismatch")
+    _check_kv(q.dtype, k_cache, v_cache, k_cache.shape[1], d, vd)
+    _need(sink is None or (sink.dtype == torch.float32 and sink.numel() == heads), "one float32 sink per head")
+    _need(turn_back is None or (turn_back.dtype == torch.float32 and turn_back.shape == (T, vd // 2, 2) and vd % 2 == 0
+                                and turn_back.is_contiguous()), "turn_back must be float32 [T, value size / 2, 2]")
     kv_heads, page_size = k_cache.shape[1], k_cache.shape[2]
     _need(block_table.dim() == 2, "block table must be [requests, pages]")
     _is_i32(block_table)
     _is_i32(seq_of_token, T)
     _is_i32(positions, T)
     _call("ix_attention_plain", _ptr(q), _ptr(k_cache), _ptr(v_cache), _i32(_dt(q)), _ptr(block_table),
-          _ptr(seq_of_token), _ptr(positions), _ptr(out), _i64(T), _i32(heads), _i32(kv_heads), _i32(d),
-          _i32(page_size), _i32(block_table.shape[1]), _f32(scale), _i32(window), _stream())
+          _ptr(seq_of_token), _ptr(positions), _ptr(out), _i64(T), _i32(heads), _i32(kv_heads), _i32(d), _i32(vd),
+          _i32(page_size), _i32(block_table.shape[1]), _f32(scale), _i32(window), _ptr(sink), _ptr(turn_back), _stream())
+
+
+def qkv_norm_rope_append(qkv: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float,
+                         cos_sin: Optional[torch.Tensor], rot_begin: int, v_cos_sin: Optional[torch.Tensor],
+                         slots: Optional[torch.Tensor], q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
+                         v_cache: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int,
+                         value_dim: int) -> None:
+    """After the q|k|v product, per token and head: an RMS norm over the head with a weight per element (q and k,
+    where `q_norm`, `k_norm` [head_dim] are given), the rotation of the 2 * cos_sin.shape[1] elements from `rot_begin`
+    on (pairs (i, i + half) within them; float32 table [T, half, 2]), the rotation of ALL of a value head by its own
+    table `v_cos_sin` [T, value_dim / 2, 2]; q goes to q_out [T, heads, head_dim], k and v to the token's slot of the
+    paged caches (keys [pages, kv_heads, page_size, head_dim], values [pages, kv_heads, value_dim, page_size])."""
+    T = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.is_cuda
+          and qkv.shape[1] >= (heads + kv_heads) * head_dim + kv_heads * value_dim, "qkv rows too short")
+    _need(q_out.shape == (T, heads, head_dim) and q_out.dtype == qkv.dtype and q_out.is_contiguous(), "q_out mismatch")
+    for w in (q_norm, k_norm):
+        _need(w is None or (w.numel() == head_dim and w.is_contiguous()), "a norm weight per element of a head")
+    half = 0
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[0] == T and cos_sin.shape[2] == 2
+              and cos_sin.is_contiguous(), "the rotation table must be float32 [T, half, 2]")
+        half = cos_sin.shape[1]
+        _need(rot_begin >= 0 and rot_begin + 2 * half <= head_dim, "the rotated part must lie within the head")
+    if v_cos_sin is not None:
+        _need(v_cos_sin.dtype == torch.float32 and v_cos_sin.shape == (T, value_dim // 2, 2) and value_dim % 2 == 0
+              and v_cos_sin.is_contiguous(), "the values' rotation table must be float32 [T, value_dim / 2, 2]")
+    page_size = 1
+    if slots is not None:
+        _check_kv(qkv.dtype, k_cache, v_cache, kv_heads, head_dim, value_dim)
+        _need(k_cache.is_contiguous() and v_cache.is_contiguous(), "the caches must be contiguous")
+        page_size = k_cache.shape[2]
+        _is_i32(slots, T)
+    wq, wk = q_norm, k_norm
+    _call("ix_qkv_norm_rope_append", qkv.data_ptr(), _i32(_dt(qkv)), _i64(qkv.stride(0)), _ptr(wq),
+          _i32(_dt(wq) if wq is not None else F32), _ptr(wk), _i32(_dt(wk) if wk is not None else F32), _f32(eps),
+          _ptr(cos_sin), _i32(rot_begin), _i32(half), _ptr(v_cos_sin), _ptr(slots), _ptr(q_out),
+          _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, _i64(T), _i32(heads),
+          _i32(kv_heads), _i32(head_dim), _i32(value_dim), _i32(page_size),
+          _i64(k_cache.shape[0] * page_size if slots is not None else 0), _stream())
+
+
+def rotate_heads(x: torch.Tensor, cos_sin: torch.Tensor, inverse: bool = False) -> None:
+    """x [T, heads, d] in place: every head's pair (i, i + d / 2) turned by the token's angle i of `cos_sin` (float32
+    [T, d / 2, 2]); `inverse` turns the other way."""
+    T, heads, d = x.shape
+    _need(x.is_contiguous() and d % 2 == 0, "x must be dense [T, heads, d] with an even d")
+    _need(cos_sin.dtype == torch.float32 and cos_sin.shape == (T, d // 2, 2) and cos_sin.is_contiguous(),
+          "the rotation table must be float32 [T, d / 2, 2]")
+    _call("ix_rotate_heads", _ptr(x), _i32(_dt(x)), _ptr(cos_sin), _i64(T), _i32(heads), _i32(d), _i32(1 if inverse else 0),
+          _stream())
 
 
 def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -1020,25 +1103,59 @@ def short_conv(x: torch.Tensor, bias: Optional[torch.Tensor], weight: torch.Tens
 
 def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor,
                dt_bias: torch.Tensor, state: torch.Tensor, rows: StepRows, out: torch.Tensor, heads: int,
-               kv_heads: int, dim: int, vdim: int) -> None:
+               kv_heads: int, dim: int, vdim: int, channel_logits: Optional[torch.Tensor] = None) -> None:
     """The gated delta rule over the rows of a step, request by request, from and to `state` (a float32 view
     [slots, >= heads * dim * vdim]).  q, k [T, kv_heads * dim], v [T, heads * vdim] (rows may be strided);
-    ab float32 [T, 2 heads]: the decay's and the step size's logits; out float32 [T, heads, vdim]."""
+    ab float32 [T, 2 heads]: the decay's and the step size's logits; out float32 [T, heads, vdim].
+    `channel_logits` float32 [T, heads * dim]: a decay per key channel from these logits, with dt_bias
+    [heads * dim]; ab is then float32 [T, heads], the step size's logits alone."""
     T = q.shape[0]
+    per = 1 if channel_logits is None else dim
     for t, n in ((q, kv_heads * dim), (k, kv_heads * dim), (v, heads * vdim)):
         _need(t.dim() == 2 and t.shape == (T, n) and t.stride(1) == 1 and t.dtype == q.dtype and t.is_cuda, "q, k or v shape")
-    _need(ab.dtype == torch.float32 and ab.shape == (T, 2 * heads) and ab.is_contiguous(), "ab must be float32 [T, 2 heads]")
+    if channel_logits is None:
+        _need(ab.dtype == torch.float32 and ab.shape == (T, 2 * heads) and ab.is_contiguous(), "ab must be float32 [T, 2 heads]")
+    else:
+        _need(ab.dtype == torch.float32 and ab.shape == (T, heads) and ab.is_contiguous(), "ab must be float32 [T, heads]")
+        _need(channel_logits.dtype == torch.float32 and channel_logits.shape == (T, heads * dim)
+              and channel_logits.is_contiguous(), "the decays' logits must be float32 [T, heads * dim]")
     _need(a_log.dtype == torch.float32 and a_log.numel() == heads and dt_bias.dtype == torch.float32
-          and dt_bias.numel() == heads, "a_log and dt_bias must be float32 [heads]")
+          and dt_bias.numel() == heads * per and dt_bias.is_contiguous(),
+          "a_log must be float32 [heads], dt_bias float32 with one number per decay")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
           and state.shape[1] >= heads * dim * vdim, "the state must be float32 [slots, >= heads * dim * vdim]")
     _need(out.dtype == torch.float32 and out.shape == (T, heads, vdim), "out must be float32 [T, heads, vdim]")
     rows.check(T)
     S = rows.q_start.numel() - 1
     _call("ix_delta_rule", q.data_ptr(), k.data_ptr(), v.data_ptr(), _i32(_dt(q)), _i64(q.stride(0)), _i64(k.stride(0)),
-          _i64(v.stride(0)), _ptr(ab), _ptr(a_log), _ptr(dt_bias), state.data_ptr(), _i64(state.stride(0)),
+          _i64(v.stride(0)), _ptr(ab), _ptr(channel_logits), _ptr(a_log), _ptr(dt_bias), state.data_ptr(), _i64(state.stride(0)),
           _ptr(rows.q_start), _ptr(rows.state_slots), _ptr(out), _i64(T), _i32(S), _i32(heads), _i32(kv_heads),
           _i32(dim), _i32(vdim), _stream())
+
+
+def matrix_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor,
+                  cap: float, state: torch.Tensor, rows: StepRows, out: torch.Tensor, heads: int, dim: int,
+                  vdim: int) -> None:
+    """The matrix memory with exponential gates over the rows of a step, request by request, from and to `state` (a
+    float32 view [slots, >= heads * dim * vdim + heads * dim + heads]: matrices, then n, then the running maxima).
+    q, k [T, heads * dim], v [T, heads * vdim] (rows may be strided); gates float32 [T, 2 heads] (input gate's logits,
+    then forget gate's), gate_bias float32 [2 heads]; out float32 [T, heads, vdim]."""
+    T = q.shape[0]
+    for t, n in ((q, heads * dim), (k, heads * dim), (v, heads * vdim)):
+        _need(t.dim() == 2 and t.shape == (T, n) and t.stride(1) == 1 and t.dtype == q.dtype and t.is_cuda, "q, k or v shape")
+    _need(gates.dtype == torch.float32 and gates.shape == (T, 2 * heads) and gates.is_contiguous(),
+          "gates must be float32 [T, 2 heads]")
+    _need(gate_bias.dtype == torch.float32 and gate_bias.numel() == 2 * heads and gate_bias.is_contiguous(),
+          "gate_bias must be float32 [2 heads]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= heads * dim * vdim + heads * dim + heads, "the state must be float32 [slots, >= matrices + n + m]")
+    _need(out.dtype == torch.float32 and out.shape == (T, heads, vdim) and out.is_contiguous(), "out must be float32 [T, heads, vdim]")
+    rows.check(T)
+    S = rows.q_start.numel() - 1
+    _call("ix_matrix_memory", q.data_ptr(), k.data_ptr(), v.data_ptr(), _i32(_dt(q)), _i64(q.stride(0)), _i64(k.stride(0)),
+          _i64(v.stride(0)), _ptr(gates), _ptr(gate_bias), _f32(cap), state.data_ptr(), _i64(state.stride(0)),
+          _ptr(rows.q_start), _ptr(rows.state_slots), _ptr(out), _i64(T), _i32(S), _i32(heads), _i32(dim), _i32(vdim),
+          _stream())
 
 
 def head_norm_gate(x: torch.Tensor, out: torch.Tensor, eps: float, weight: Optional[torch.Tensor] = None,
@@ -1202,9 +1319,9 @@ def tanh_(x: torch.Tensor) -> None:
 # ---- attention over a compressed cache ------------------------------------------------------------------------------
 def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, norm_w: torch.Tensor, eps: float,
                    cos_sin: Optional[torch.Tensor], slots: Optional[torch.Tensor], cache: torch.Tensor, heads: int,
-                   rot_dim: int, rank: int) -> None:
+                   rot_dim: int, rank: int, halves: bool = False) -> None:
     """Per token: the last `rot_dim` numbers of every head of q [T, heads * q_dim] are rotated in place (pairs
-    (2i, 2i + 1), i < cos_sin.shape[1]; float32 table [T, pairs, 2]); the first `rank` numbers of the dkv row pass an
+    (2i, 2i + 1), i < cos_sin.shape[1]; float32 table [T, pairs, 2]; with `halves` the pairs (i, i + pairs)); the first `rank` numbers of the dkv row pass an
     RMS norm with `norm_w` (float32 sums), its last rot_dim are rotated likewise, and [c | kr] goes to row slots[t] of
     `cache` [pages, 1, page_size, rank + rot_dim]."""
     T = q.shape[0]
@@ -1225,7 +1342,7 @@ def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, norm_w: torch.Tensor, eps
         _is_i32(slots, T)
     _call("ix_latent_prepare", q.data_ptr(), _i64(q.stride(0)), dkv.data_ptr(), _i64(dkv.stride(0)), _i32(_dt(q)), _ptr(norm_w),
           _i32(_dt(norm_w)), _f32(eps), _ptr(cos_sin), _i32(pairs), _ptr(slots), _ptr(cache), _i64(T), _i32(heads),
-          _i32(q_dim), _i32(rot_dim), _i32(rank), _stream())
+          _i32(q_dim), _i32(rot_dim), _i32(rank), _i32(1 if halves else 0), _stream())
 
 
 def _head_rows(t: torch.Tensor, tokens: int, heads: int, n: int, what: str):
@@ -1237,9 +1354,9 @@ def _head_rows(t: torch.Tensor, tokens: int, heads: int, n: int, what: str):
 
 def latent_attention_plain(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
                            seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, rank: int,
-                           rot_dim: int, scale: float) -> None:
+                           rot_dim: int, scale: float, window: int = 0) -> None:
     """Causal attention of queries [token, head] over cached rows [c | kr]: score = (q_lat . c + q_rot . kr) * scale,
-    softmax in float32, out = sum of weights * c.  q_lat, out [token, head, rank] and q_rot [token, head, rot_dim] are
+    softmax in float32, out = sum of weights * c.  `window` W > 0: a query reads its own and the W - 1 rows before.  q_lat, out [token, head, rank] and q_rot [token, head, rot_dim] are
     views with any token and head strides; cache [pages, 1, page_size, rank + rot_dim]."""
     T, heads = q_lat.shape[0], q_lat.shape[1]
     ql_t, ql_h = _head_rows(q_lat, T, heads, rank, "q_lat")
@@ -1255,7 +1372,7 @@ def latent_attention_plain(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torc
     _call("ix_latent_attention_plain", q_lat.data_ptr(), _i64(ql_t), _i64(ql_h), q_rot.data_ptr(), _i64(qr_t), _i64(qr_h),
           _ptr(cache), _i32(_dt(q_lat)), _ptr(block_table), _ptr(seq_of_token), _ptr(positions), out.data_ptr(),
           _i64(o_t), _i64(o_h), _i64(T), _i32(heads), _i32(rank), _i32(rot_dim), _i32(cache.shape[2]),
-          _i32(block_table.shape[1]), _f32(scale), _stream())
+          _i32(block_table.shape[1]), _f32(scale), _i32(window), _stream())
 
 
 LATENT_MFMA_MAX_SPLITS = 32
@@ -1284,7 +1401,7 @@ def latent_mfma_splits(tokens: int, heads: int) -> int:
 def latent_attention_mfma(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
                           seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, rank: int,
                           rot_dim: int, scale: float, one_token_each: bool = False, n_splits: int = 1,
-                          work: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> None:
+                          work: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, window: int = 0) -> None:
     """`latent_attention_plain` on the matrix cores (see `latent_mfma_fits`).  `one_token_each`: every request brings
     one token; its keys may then be cut into `n_splits` slices, with `work` = float32 ([T * heads * n_splits, rank],
     [T * heads * n_splits, 2]) and a contiguous `out` [T, heads, rank]."""
@@ -1310,4 +1427,5 @@ def latent_attention_mfma(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch
     _call("ix_latent_attention_mfma", q_lat.data_ptr(), _i64(ql_t), _i64(ql_h), q_rot.data_ptr(), _i64(qr_t), _i64(qr_h),
           _ptr(cache), _ptr(block_table), _ptr(seq_of_token), _ptr(positions), out.data_ptr(), _i64(o_t), _i64(o_h),
           _ptr(part_o), _ptr(part_ml), _i32(n_splits), _i64(T), _i32(heads), _i32(rank), _i32(rot_dim),
-          _i32(cache.shape[2]), _i32(block_table.shape[1]), _f32(scale), _i32(1 if one_token_each else 0), _stream())
+          _i32(cache.shape[2]), _i32(block_table.shape[1]), _f32(scale), _i32(1 if one_token_each else 0), _i32(window),
+          _stream())

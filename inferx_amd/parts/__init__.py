@@ -1,7 +1,7 @@
 """Parts a layer is put together from; importing this package registers the built-in ones."""
 from .base import (Block, BranchGain, CacheArray, CacheNeed, Embedding, FeedForward, Head, LazyDelta, LazyNorm, Mixer, Norm, ParamSpec, Part,
                    PositionEncoding, ScaledDelta, StateNeed, TokenShift, build_block, build_part, register_part, resolve_delta, resolve_input)
-from . import norm, rope, dense_mlp, attention, moe, block, embedding, dyt, gain_shift, attention_talk, delta_rule, attention_diff, latent_attention, linear_state  # noqa: F401  (registration)
+from . import norm, rope, dense_mlp, attention, moe, block, embedding, dyt, gain_shift, attention_talk, delta_rule, attention_diff, latent_attention, linear_state, matrix_memory  # noqa: F401  (registration)
 from .model import DecoderModel, build_model
 
 __all__ = ["Block", "CacheArray", "CacheNeed", "Embedding", "Head", "FeedForward", "Mixer", "Norm", "ParamSpec", "Part", "PositionEncoding",

@@ -6,6 +6,14 @@ src/model/qwen2.cc:1368-1403); one kernel adds the bias, rotates q and k and
 appends k, v to the cache (:920-969); attention reads keys [start, p] through
 the request's block table (layers.cu:256-318, window :329-407); then the output
 product (:1026-1027).
+
+Options beside that, each a parameter: `qk_norm` (queries and keys pass an RMS norm per head, with a weight per
+element that the heads share, before they are rotated), `sink` (a learned number per head whose exponential joins
+the softmax's denominator: no key, no value, not scaled, counted once), `value_dim` (values of another size than
+keys) and `value_position` (a position encoding over ALL of a value head: the value of position j is cached rotated
+by j, and every head's weighted sum at position i is rotated back by i, so that what a query receives depends on
+i - j only).  With any of these the step after the product is `ops.qkv_norm_rope_append`; with a sink, rotated values
+or values of another size the attention itself is the plain kernel.
 """
 from __future__ import annotations
 
@@ -25,7 +33,9 @@ class PagedAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, qkv_bias: bool = True,
                  out_bias: bool = False, window: int = 0, scale: Optional[float] = None,
-                 position: Optional[PartSpec] = None, init_std: float = 0.02):
+                 position: Optional[PartSpec] = None, init_std: float = 0.02, value_dim: Optional[int] = None,
+                 qk_norm: bool = False, qk_norm_eps: float = 1e-6, sink: bool = False,
+                 value_position: Optional[PartSpec] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
         if head_dim % 2 or head_dim > 256:
@@ -44,7 +54,19 @@ class PagedAttention(Mixer):
             if begin < 0 or dim <= 0 or dim % 2 or begin + dim > self.head_dim:
                 raise ValueError(f"the position encoding rotates elements {begin} to {begin + dim} of heads of "
                                  f"{self.head_dim}: an even number of elements within the head is needed")
-        self.w_qkv = self.b_qkv = self.w_out = self.b_out = None
+        self.value_dim = self.head_dim if value_dim is None else int(value_dim)
+        self.qk_norm, self.qk_norm_eps, self.has_sink = bool(qk_norm), float(qk_norm_eps), bool(sink)
+        self.value_position = build_part("position", value_position) if value_position is not None else None
+        if self.value_dim <= 0 or self.value_dim > 256:
+            raise ValueError(f"value_dim {self.value_dim} must be between 1 and 256")
+        if self.value_position is not None and (getattr(self.value_position, "begin", 0) != 0 or
+                                                getattr(self.value_position, "rotary_dim", 0) != self.value_dim):
+            raise ValueError("the values' position encoding must rotate all of a value head")
+        # the step after the product that knows norms per head, rotated values and values of another size
+        self.general = self.qk_norm or self.value_position is not None or self.value_dim != self.head_dim
+        if self.general and self.qkv_bias:
+            raise ValueError("biases on q, k, v do not go with norms per head, rotated values or values of another size")
+        self.w_qkv = self.b_qkv = self.w_out = self.b_out = self.q_norm = self.k_norm = self.sink = None
 
     @property
     def q_dim(self) -> int:
@@ -54,16 +76,30 @@ class PagedAttention(Mixer):
     def kv_dim(self) -> int:
         return self.num_kv_heads * self.head_dim
 
+    @property
+    def v_dim(self) -> int:
+        return self.num_kv_heads * self.value_dim
+
+    @property
+    def out_dim(self) -> int:
+        return self.num_heads * self.value_dim
+
     def cache_need(self) -> CacheNeed:
-        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window,
+                                         None if self.value_dim == self.head_dim else self.value_dim)
 
     def subparts(self):
-        return [self.position]
+        return [self.position, self.value_position]
 
     def param_specs(self) -> List[ParamSpec]:
         H, s = self.hidden_size, self.init_std
         specs = [ParamSpec("q_proj.weight", (self.q_dim, H), std=s), ParamSpec("k_proj.weight", (self.kv_dim, H), std=s),
-                 ParamSpec("v_proj.weight", (self.kv_dim, H), std=s), ParamSpec("o_proj.weight", (H, self.q_dim), std=s)]
+                 ParamSpec("v_proj.weight", (self.v_dim, H), std=s), ParamSpec("o_proj.weight", (H, self.out_dim), std=s)]
+        if self.qk_norm:
+            specs += [ParamSpec("q_norm.weight", (self.head_dim,), std=0.1, mean=1.0),
+                      ParamSpec("k_norm.weight", (self.head_dim,), std=0.1, mean=1.0)]
+        if self.has_sink:
+            specs.append(ParamSpec("sink", (self.num_heads,), std=1.0))
         if self.qkv_bias:
             specs += [ParamSpec("q_proj.bias", (self.q_dim,), std=s), ParamSpec("k_proj.bias", (self.kv_dim,), std=s),
                       ParamSpec("v_proj.bias", (self.kv_dim,), std=s)]
@@ -76,8 +112,13 @@ class PagedAttention(Mixer):
         self.b_qkv = stack_rows([tensors[f"{n}_proj.bias"] for n in "qkv"]) if self.qkv_bias else None
         self.w_out = tensors["o_proj.weight"].contiguous()
         self.b_out = tensors["o_proj.bias"].contiguous() if self.out_bias else None
-        if self.position is not None:
-            self.position.bind({}, rt)
+        if self.qk_norm:
+            self.q_norm, self.k_norm = tensors["q_norm.weight"].contiguous(), tensors["k_norm.weight"].contiguous()
+        if self.has_sink:
+            self.sink = tensors["sink"].to(torch.float32).contiguous()
+        for position in (self.position, self.value_position):
+            if position is not None:
+                position.bind({}, rt)
 
     def capture_plan(self, ctx, requests: int, longest: int) -> None:
         """The query tiles of a step of one token per request never change: tile i = request i, row i, one query;
@@ -94,6 +135,15 @@ class PagedAttention(Mixer):
         table = self.position.prepare(ctx) if self.position is not None else None
         q = rt.empty((T, self.num_heads, self.head_dim))
         writes = cache.writes
+        if self.general:
+            turn = self.value_position.prepare(ctx) if self.value_position is not None else None
+            ops.qkv_norm_rope_append(rt.linear(x, self.w_qkv), self.q_norm, self.k_norm, self.qk_norm_eps, table,
+                                     self.rotated[0], turn, ctx.slots[cache.group] if writes else None, q,
+                                     cache.k if writes else None, cache.v if writes else None, self.num_heads,
+                                     self.num_kv_heads, self.head_dim, self.value_dim)
+            out = rt.empty((T, self.num_heads, self.value_dim))
+            self.attend(ctx, q, cache, out, turn)
+            return rt.linear(out.view(T, self.out_dim), self.w_out)
         epilogue = (self.b_qkv, table, ctx.slots[cache.group] if writes else None, q, cache.k if writes else None,
                     cache.v if writes else None, self.num_heads, self.num_kv_heads, self.head_dim)
         whole = table is None or self.rotated == (0, self.head_dim)
@@ -109,12 +159,14 @@ class PagedAttention(Mixer):
             ops.add_bias(y, self.b_out)
         return y
 
-    def attend(self, ctx, q, cache, out) -> None:
+    def attend(self, ctx, q, cache, out, turn_back=None) -> None:
         """bfloat16 with pages and heads in multiples of 16: the matrix-core kernels (the one that shares keys through
         LDS for the prompt portions of a step, the wavefront-level one for requests that bring few tokens and for
-        steps of one token per request); else the plain one."""
+        steps of one token per request); else the plain one, which also knows a sink, values of another size than
+        keys and a result that is rotated back (`turn_back`: the table of the query's angles)."""
         page_size = cache.k.shape[2]
-        if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0:
+        special = self.sink is not None or turn_back is not None or self.value_dim != self.head_dim
+        if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0 and not special:
             T = ctx.num_tokens
             if not ctx.one_token_each:  # some request brings more than one token: the step's plan says who goes where
                 lds_fits = self.head_dim <= 128 and page_size & (page_size - 1) == 0
@@ -150,7 +202,7 @@ class PagedAttention(Mixer):
                                n_splits, work, self.scale, self.window, tile, prefetch=True, grouped=grouped)
         else:
             ops.attention_plain(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.seq_of_token, ctx.positions,
-                                out, self.scale, self.window)
+                                out, self.scale, self.window, self.sink, turn_back)
 
 
 # ---- the wavefront-level kernel (ops.attention_mfma)

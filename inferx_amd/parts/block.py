@@ -14,6 +14,7 @@ import torch
 from .. import ops
 from .base import Block, LazyDelta, LazyNorm, register_part, resolve_delta
 from .dense_mlp import BiasedDelta
+from .gain_shift import WeightedSum
 from .norm import NormedDelta
 
 
@@ -160,7 +161,49 @@ class ParallelBlock(Block):
         return BranchSum(resolve_delta(ctx, a), self.feed_forward.forward(ctx, x))
 
 
+class PreNormBranchesBlock(Block):
+    """`prenorm` whose mixer may have a second mixer beside it, both reading the one norm, each with a constant gain:
+
+        x = norm1(h + pending);  h += ga * mixer(x) + gb * second_mixer(x);  pending = feed_forward(norm2(h))
+
+    `second_mixer`, the gains (kind "gain", parts with a `factor`) and the feed-forward with its norm may be left
+    out; without a feed-forward the mixers' result stays pending for the next layer.  Each mixer keeps pages or
+    state of its own (`caches` by part name)."""
+
+    graph_safe = True
+    part_kinds = {"mixer": "mixer", "second_mixer": "mixer", "mixer_gain": "gain", "second_mixer_gain": "gain",
+                  "feed_forward": "feed_forward", "mixer_norm": "norm", "feed_forward_norm": "norm"}
+    optional_parts = ("second_mixer", "mixer_gain", "second_mixer_gain", "feed_forward", "feed_forward_norm")
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        if (self.feed_forward is None) != (self.feed_forward_norm is None):
+            raise KeyError("a feed-forward and the norm before it come together or not at all")
+        if self.second_mixer is None and self.second_mixer_gain is not None:
+            raise KeyError("a gain for a second mixer that is not there")
+        for gain in (self.mixer_gain, self.second_mixer_gain):
+            if gain is not None and not hasattr(gain, "factor"):
+                raise KeyError("the gains of this arrangement are constants (parts with a `factor`)")
+
+    def forward(self, ctx, h, pending, caches):
+        x = self.mixer_norm.forward(ctx, h, pending)
+        a = self.mixer.forward(ctx, x, caches.get("mixer"))
+        fa = 1.0 if self.mixer_gain is None else self.mixer_gain.factor
+        if self.second_mixer is not None:
+            b = self.second_mixer.forward(ctx, x, caches.get("second_mixer"))
+            fb = 1.0 if self.second_mixer_gain is None else self.second_mixer_gain.factor
+            a = WeightedSum([(resolve_delta(ctx, a), fa), (resolve_delta(ctx, b), fb)])
+        elif fa != 1.0:
+            a = WeightedSum([(resolve_delta(ctx, a), fa)])
+        if self.feed_forward is None:
+            return a
+        if self.feed_forward.takes_lazy_norm:
+            return self.feed_forward.forward(ctx, LazyNorm(self.feed_forward_norm, h, a))
+        return self.feed_forward.forward(ctx, self.feed_forward_norm.forward(ctx, h, a))
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "prenorm_branches", PreNormBranchesBlock)
 register_part("block", "parallel", ParallelBlock)
 register_part("block", "sandwich_norm", SandwichNormBlock)
 register_part("block", "prenorm_gained", GainedPreNormBlock)

@@ -67,4 +67,38 @@ class DenseMlp(FeedForward):
         return y if self.b_down is None else BiasedDelta(y, self.b_down)
 
 
+class PolyNormMlp(FeedForward):
+    """A feed-forward without a gate whose activation blends the normalised first three powers of its input:
+
+        z = x . Wup^T;   y = (a N(z) + b N(z^2) + c N(z^3) + e) . Wdown^T,   N(v) = v / sqrt(mean(v^2) + eps)
+
+    with the powers taken element by element and the four numbers a, b, c, e learned (`act`).  The sums of squares
+    and the blend are float32."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, width: int, norm_eps: float = 1e-6, init_std: float = 0.02):
+        self.hidden_size, self.width = int(hidden_size), int(width)
+        self.norm_eps, self.init_std = float(norm_eps), float(init_std)
+        self.w_up = self.w_down = self.coef = None
+
+    def param_specs(self) -> List[ParamSpec]:
+        H, I, s = self.hidden_size, self.width, self.init_std
+        return [ParamSpec("up_proj.weight", (I, H), std=s), ParamSpec("down_proj.weight", (H, I), std=s),
+                ParamSpec("act", (4,), std=0.3, mean=0.3)]
+
+    def bind(self, tensors, rt) -> None:
+        self.w_up, self.w_down = tensors["up_proj.weight"].contiguous(), tensors["down_proj.weight"].contiguous()
+        self.coef = tensors["act"].to(torch.float32).contiguous()
+
+    def forward(self, ctx, x):
+        from .. import ops
+        rt = ctx.rt
+        z = rt.linear(x, self.w_up)
+        y = rt.empty(tuple(z.shape))
+        ops.polynorm(z, self.coef, y, self.norm_eps)
+        return rt.linear(y, self.w_down)
+
+
 register_part("feed_forward", "dense_mlp", DenseMlp)
+register_part("feed_forward", "polynorm_mlp", PolyNormMlp)

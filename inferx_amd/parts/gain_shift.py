@@ -14,7 +14,7 @@ from typing import List
 import torch
 
 from .. import ops
-from .base import BranchGain, ParamSpec, ScaledDelta, StateNeed, TokenShift, register_part, resolve_delta
+from .base import BranchGain, LazyDelta, ParamSpec, ScaledDelta, StateNeed, TokenShift, register_part, resolve_delta
 
 
 class ChannelGain(BranchGain):
@@ -34,6 +34,35 @@ class ChannelGain(BranchGain):
         if isinstance(delta, ScaledDelta):  # a gain on a gain: one vector does both
             return ScaledDelta(delta.tensor, delta.gain * self.weight)
         return ScaledDelta(delta, self.weight)
+
+
+class ConstantGain(BranchGain):
+    """A branch's result times ONE fixed number (a constant of the configuration, no tensor).  Where two branches
+    meet, the arrangement forms fa * a + fb * b in one pass (`WeightedSum`); alone it is a `WeightedSum` of one."""
+
+    graph_safe = True
+
+    def __init__(self, factor: float):
+        self.factor = float(factor)
+
+    def apply(self, delta):
+        return WeightedSum([(delta, self.factor)])
+
+
+class WeightedSum(LazyDelta):
+    """fa * a + fb * b of one or two branches' results (tensors of the run's type), not formed yet; whoever adds it
+    to the stream gets the float32 sum, formed in one pass."""
+
+    def __init__(self, terms):
+        if not 1 <= len(terms) <= 2:
+            raise ValueError("a weighted sum of one or two branches")
+        self.terms = list(terms)
+
+    def materialize(self, ctx):
+        (a, fa), (b, fb) = self.terms[0], (self.terms[1] if len(self.terms) == 2 else (None, 0.0))
+        out = ctx.rt.empty(tuple(a.shape), torch.float32)
+        ops.weighted_sum(a, fa, b, fb, out)
+        return out
 
 
 class PreviousTokenShift(TokenShift):
@@ -64,4 +93,5 @@ class PreviousTokenShift(TokenShift):
 
 
 register_part("gain", "channel_gain", ChannelGain)
+register_part("gain", "constant_gain", ConstantGain)
 register_part("shift", "previous_token", PreviousTokenShift)

@@ -11,7 +11,11 @@ maps, and one rotated key part that all heads share.
 
 Only [c | kr] is kept per token (`CacheNeed` of one array, one "head" of rank + rot_dim numbers), whatever the
 number of heads.  The rotation pairs element 2i with 2i + 1 over the first `rotary_dim` numbers of the rotated part
-(the position encoding's table by pair; the rest of the part passes).  Norm, angles, scores and softmax are float32.
+(the position encoding's table by pair; the rest of the part passes); with `pairing` "halves" it pairs element i with
+i + rotary_dim / 2 instead.  Norm, angles, scores and softmax are float32.
+
+Options: `window` W (a query reads its own row and the W - 1 before it; older pages are given back), and `gate`
+(the heads' results times sigmoid(x . Wg^T), element by element, before the last product).
 """
 from __future__ import annotations
 
@@ -30,7 +34,7 @@ class LatentAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int,
                  scale: Optional[float] = None, norm_eps: float = 1e-6, position: Optional[PartSpec] = None,
-                 init_std: float = 0.02):
+                 init_std: float = 0.02, pairing: str = "pairs", window: int = 0, gate: bool = False):
         if min(num_heads, head_dim, value_dim, kv_rank) <= 0 or rot_dim < 0:
             raise ValueError("heads, head_dim, value_dim and kv_rank must be positive, rot_dim not negative")
         if kv_rank > 1024 or rot_dim > 64 + 1024 - kv_rank:
@@ -41,6 +45,9 @@ class LatentAttention(Mixer):
         self.q_dim = self.head_dim + self.rot_dim
         self.scale = float(scale) if scale is not None else self.q_dim ** -0.5
         self.norm_eps, self.init_std = float(norm_eps), float(init_std)
+        if pairing not in ("pairs", "halves") or window < 0:
+            raise ValueError(f"pairing {pairing!r} (pairs or halves), window {window} (not negative)")
+        self.halves, self.window, self.has_gate = pairing == "halves", int(window), bool(gate)
         self.position = build_part("position", position) if position is not None else None
         if self.position is not None:
             dims = int(getattr(self.position, "rotary_dim", 0))
@@ -50,7 +57,7 @@ class LatentAttention(Mixer):
         self.w_in = self.w_uk = self.w_uv_t = self.w_out = self.norm_weight = None
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed((CacheArray("latent", 1, self.kv_rank + self.rot_dim),))
+        return CacheNeed((CacheArray("latent", 1, self.kv_rank + self.rot_dim),), self.window)
 
     def subparts(self):
         return [self.position]
@@ -62,11 +69,13 @@ class LatentAttention(Mixer):
                 ParamSpec("dkv_norm.weight", (self.kv_rank,), init="ones"),
                 ParamSpec("uk.weight", (H * self.head_dim, self.kv_rank), std=s),
                 ParamSpec("uv.weight", (H * self.value_dim, self.kv_rank), std=s),
-                ParamSpec("o.weight", (W, H * self.value_dim), std=s)]
+                ParamSpec("o.weight", (W, H * self.value_dim), std=s)] + (
+                    [ParamSpec("g.weight", (H * self.value_dim, W), std=s)] if self.has_gate else [])
 
     def bind(self, tensors, rt) -> None:
         H = self.num_heads
-        self.w_in = stack_rows([tensors["q.weight"], tensors["dkv.weight"]])
+        self.w_in = stack_rows([tensors["q.weight"], tensors["dkv.weight"]] +
+                               ([tensors["g.weight"]] if self.has_gate else []))
         self.w_uk = tensors["uk.weight"].contiguous().view(H, self.head_dim, self.kv_rank)
         self.w_uv_t = tensors["uv.weight"].view(H, self.value_dim, self.kv_rank).transpose(1, 2).contiguous()
         self.w_out = tensors["o.weight"].contiguous()
@@ -78,10 +87,11 @@ class LatentAttention(Mixer):
         rt, T, H = ctx.rt, x.shape[0], self.num_heads
         table = self.position.prepare(ctx) if self.position is not None else None
         proj = rt.linear(x, self.w_in)  # q of all heads | d
-        q, dkv = proj[:, :H * self.q_dim], proj[:, H * self.q_dim:]
+        q, dkv = proj[:, :H * self.q_dim], proj[:, H * self.q_dim:H * self.q_dim + self.kv_rank + self.rot_dim]
         latent = cache.arrays["latent"]
         ops.latent_prepare(q, dkv, self.norm_weight, self.norm_eps, table,
-                           ctx.slots[cache.group] if cache.writes else None, latent, H, self.rot_dim, self.kv_rank)
+                           ctx.slots[cache.group] if cache.writes else None, latent, H, self.rot_dim, self.kv_rank,
+                           self.halves)
         q3 = q.unflatten(1, (H, self.q_dim))
         q_lat = torch.bmm(q3[:, :, :self.head_dim].transpose(0, 1), self.w_uk)  # [H, T, rank]
         if ctx.one_token_each:  # (the slices of a token's keys meet in a contiguous [T, H, rank])
@@ -91,13 +101,15 @@ class LatentAttention(Mixer):
         self.attend(ctx, q_lat.transpose(0, 1), q3[:, :, self.head_dim:], cache, o_lat.transpose(0, 1))
         y = rt.empty((T, H * self.value_dim))
         torch.bmm(o_lat, self.w_uv_t, out=y.view(T, H, self.value_dim).transpose(0, 1))
+        if self.has_gate:
+            ops.sigmoid_gate(y, proj[:, H * self.q_dim + self.kv_rank + self.rot_dim:])
         return rt.linear(y, self.w_out)
 
     def attend(self, ctx, q_lat, q_rot, cache, out) -> None:
         latent, table = cache.arrays["latent"], ctx.block_tables[cache.group]
         if not ops.latent_mfma_fits(q_lat, q_rot, out, self.kv_rank, self.rot_dim):  # float32 runs, other sizes
             ops.latent_attention_plain(q_lat, q_rot, latent, table, ctx.seq_of_token, ctx.positions, out, self.kv_rank,
-                                       self.rot_dim, self.scale)
+                                       self.rot_dim, self.scale, self.window)
             return
         rt, T, H = ctx.rt, q_lat.shape[0], self.num_heads
         splits, work = 1, None
@@ -106,7 +118,7 @@ class LatentAttention(Mixer):
             if splits > 1:
                 work = (rt.empty((T * H * splits, self.kv_rank), torch.float32), rt.empty((T * H * splits, 2), torch.float32))
         ops.latent_attention_mfma(q_lat, q_rot, latent, table, ctx.seq_of_token, ctx.positions, out, self.kv_rank,
-                                  self.rot_dim, self.scale, ctx.one_token_each, splits, work)
+                                  self.rot_dim, self.scale, ctx.one_token_each, splits, work, self.window)
 
 
 register_part("mixer", "latent_attention", LatentAttention)

@@ -16,10 +16,13 @@ from .base import LazyDelta, Norm, ParamSpec, register_part
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, width: int, eps: float, scalar: bool = False):
+    def __init__(self, width: int, eps: float, scalar: bool = False, groups: int = 1):
         """`scalar`: the weight is ONE number for all coordinates (a tensor without dimensions), spread over the
-        width when it is bound, so that every kernel that applies an RMS norm takes it as it is."""
-        self.width, self.eps, self.scalar = int(width), float(eps), bool(scalar)
+        width when it is bound, so that every kernel that applies an RMS norm takes it as it is.  `groups`: the
+        width is cut into that many equal consecutive runs, and each is divided by its own root mean square."""
+        self.width, self.eps, self.scalar, self.groups = int(width), float(eps), bool(scalar), int(groups)
+        if self.groups < 1 or self.width % self.groups:
+            raise ValueError(f"{groups} groups do not divide a width of {width}")
         self.weight = None
 
     def param_specs(self) -> List[ParamSpec]:
@@ -30,7 +33,8 @@ class RMSNorm(Norm):
         self.weight = w.reshape(1).expand(self.width).contiguous() if self.scalar else w.contiguous()
 
     def rms_operands(self):
-        return self.weight, self.eps
+        # (a norm in groups is not the plain one that other kernels know how to apply on their way)
+        return (self.weight, self.eps) if self.groups == 1 else None
 
     def forward(self, ctx, h, delta=None, rows=None):
         """h [T, width] float32 is updated in place with `delta` (unless `rows`
@@ -38,10 +42,10 @@ class RMSNorm(Norm):
         n = h.shape[0] if rows is None else rows.numel()
         out = ctx.rt.empty((n, self.width))
         if isinstance(delta, LazyDelta):
-            if delta.add_rmsnorm(ctx, h, self.weight, self.eps, rows, out):
+            if self.groups == 1 and delta.add_rmsnorm(ctx, h, self.weight, self.eps, rows, out):
                 return out
             delta = delta.materialize(ctx)
-        ops.add_rmsnorm(h, delta, self.weight, out, self.eps, rows)
+        ops.add_rmsnorm(h, delta, self.weight, out, self.eps, rows, self.groups)
         return out
 
 
