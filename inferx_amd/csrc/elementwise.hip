@@ -633,7 +633,7 @@ extern "C" int ix_add_branches(float* h, const void* a, const void* b, int dtype
 //   out = a N(z) + b N(z^2) + c N(z^3) + e,   N(v) = v / sqrt(mean(v^2) + eps)   (powers element by element)
 // The three sums of squares (of z, z^2, z^3) and the blend are float32; coef holds a, b, c, e.
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 polynorm_kernel(const T* __restrict__ z, const void* __restrict__ coef, int c_dtype, T* __restrict__ out,
                 int64_t width, float eps) {
   __shared__ float red[16];

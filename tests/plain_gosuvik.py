@@ -38,6 +38,17 @@ def bfloat16(x):
     return x.to(torch.bfloat16).to(F)
 
 
+def jittered(seed):
+    """Another sample of what 16-bit storage does: x moved at random by up to one part in 512 (as much as the rounding
+    itself), then rounded to bfloat16.  (An engine rounds at other places than this model; several samples show better
+    how far rounding alone can move a badly conditioned position.)"""
+    g = torch.Generator().manual_seed(seed)
+
+    def store(x):
+        return bfloat16(x * (1.0 + (torch.rand(x.shape, generator=g, dtype=F) * 2.0 - 1.0) / 512.0))
+    return store
+
+
 _S = exact  # what keeping an activation between two operations does to it (`forward(store=...)` sets it)
 
 
@@ -255,11 +266,12 @@ def layer_order(cfg):
     return list(range(loop["start"])) + body * loop["times"] + list(range(loop["stop"], n))
 
 
-def forward(cfg, weights, tokens, store=exact, experts=None, trace=None, chosen=None):
+def forward(cfg, weights, tokens, store=exact, experts=None, trace=None, chosen=None, scores=None):
     """Logits [T, vocab] of one sequence from its start.  `weights`: name -> tensor (any float type).  `store`: what
     keeping an activation does (`bfloat16` for a 16-bit engine).  `trace`: a list that receives the stream after every
     layer run.  `experts`: per (layer run with experts) the experts [T, top] to use instead of the router's choice;
-    `chosen`: a list that receives the router's own choice per such run."""
+    `chosen`: a list that receives the router's own choice per such run, `scores` one that receives the router's
+    scores [T, experts]."""
     global _S
     _S = store
     try:
@@ -288,6 +300,8 @@ def forward(cfg, weights, tokens, store=exact, experts=None, trace=None, chosen=
                 else:
                     if chosen is not None:
                         chosen.append(route(x, fw, f)[0])
+                    if scores is not None:
+                        scores.append(torch.softmax(x @ fw["router"].T, dim=-1))
                     h = h + experts_mlp(x, fw, f, None if experts is None else experts[run])
                     run += 1
             if trace is not None:
