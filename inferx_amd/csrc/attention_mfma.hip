@@ -44,7 +44,12 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
                  const int32_t* __restrict__ tile_q0, const int32_t* __restrict__ tile_rows,
                  const int32_t* __restrict__ positions, __bf16* __restrict__ out, float* __restrict__ part_o,
                  float* __restrict__ part_ml, int n_tiles, int n_splits, int heads, int kv_heads, int page_size,
-                 int max_blocks, float scale_log2, int window, int page_shift) {
+                 int max_blocks, float scale_log2, int window, int page_shift, const float* __restrict__ sink,
+                 const float2* __restrict__ turn_back) {
+  // sink (one float per head, or null): exp(sink) joins the softmax's denominator, with no key and no value, not
+  // scaled, once: the first slice's running maximum starts there with a sum of one.  turn_back ((cos, sin) per token
+  // and pair, [tokens][D / 2], or null; D a multiple of 32): the result is rotated by minus these angles, element i
+  // with i + D / 2, which a lane holds both of.
   constexpr int D = 16 * NB;
   constexpr int NC = (NB + 1) / 2;  // 32-wide chunks of the head dimension
   const int lane = threadIdx.x & 63;
@@ -90,8 +95,9 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
   float m[QT], lsum[QT];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    m[t] = -INFINITY;
-    lsum[t] = 0.f;
+    const bool sunk = sink != nullptr && split == 0;
+    m[t] = sunk ? sink[head] * 1.4426950408889634f : -INFINITY;
+    lsum[t] = (sunk && g == 0) ? 1.f : 0.f;  // (a column's sum is spread over its four lanes)
 #pragma unroll
     for (int b = 0; b < NB; ++b) o[t][b] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -258,6 +264,19 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
     const int64_t token = tq0 + (GQ ? 0 : 16 * t + n);
     if (n_splits == 1) {
       const float inv = 1.0f / l;
+      if constexpr (NB % 2 == 0) {
+        if (turn_back) {
+#pragma unroll
+          for (int b = 0; b < NB / 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float2 c = turn_back[token * (D / 2) + 16 * b + 4 * g + i];
+              const float u = o[t][b][i], w = o[t][b + NB / 2][i];
+              o[t][b][i] = u * c.x + w * c.y;
+              o[t][b + NB / 2][i] = w * c.x - u * c.y;
+            }
+        }
+      }
       __bf16* dst = out + (token * heads + head) * D + 4 * g;
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
@@ -284,7 +303,7 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
 // sums its columns with independent loads.
 __global__ void __launch_bounds__(128)
 attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, __bf16* __restrict__ out,
-                    int n_splits, int head_dim) {
+                    int n_splits, int head_dim, int heads, const float2* __restrict__ turn_back) {
   __shared__ float wgt[256];
   __shared__ float inv_l;
   const int64_t th = blockIdx.x;  // token * heads + head
@@ -305,6 +324,21 @@ attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ 
   }
   __syncthreads();
   const float* po = part_o + th * n_splits * head_dim;
+  if (turn_back) {  // the result rotated by minus the token's angles: a thread takes element d and d + head_dim / 2
+    const int half = head_dim / 2;
+    for (int d = threadIdx.x; d < half; d += blockDim.x) {
+      float u = 0.f, w = 0.f;
+#pragma unroll 8
+      for (int s = 0; s < n_splits; ++s) {
+        u += wgt[s] * po[s * head_dim + d];
+        w += wgt[s] * po[s * head_dim + half + d];
+      }
+      const float2 c = turn_back[(th / heads) * half + d];
+      out[th * head_dim + d] = (__bf16)((u * c.x + w * c.y) * inv_l);
+      out[th * head_dim + half + d] = (__bf16)((w * c.x - u * c.y) * inv_l);
+    }
+    return;
+  }
   for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
     float acc = 0.f;
 #pragma unroll 8
@@ -314,9 +348,9 @@ attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ 
 }
 
 int ix_attention_combine(const float* part_o, const float* part_ml, void* out, int64_t tokens, int heads,
-                         int n_splits, int head_dim, hipStream_t stream) {
+                         int n_splits, int head_dim, hipStream_t stream, const float* turn_back) {
   hipLaunchKernelGGL(attn_combine_kernel, dim3(static_cast<unsigned>(tokens * heads)), dim3(128), 0, stream, part_o,
-                     part_ml, (__bf16*)out, n_splits, head_dim);
+                     part_ml, (__bf16*)out, n_splits, head_dim, heads, reinterpret_cast<const float2*>(turn_back));
   return ix_check_launch("ix_attention_combine");
 }
 
@@ -325,7 +359,7 @@ static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void
                         const int32_t* table, const int32_t* tile_seq, const int32_t* tile_q0,
                         const int32_t* tile_rows, const int32_t* positions, void* out, float* part_o, float* part_ml,
                         int n_tiles, int n_splits, int heads, int kv_heads, int page_size, int max_blocks,
-                        float scale_log2, int window) {
+                        float scale_log2, int window, const float* sink, const float* turn_back) {
   int page_shift = -1;  // log2 of the page size if it is a power of two
   for (int b = 4; b < 31; ++b)
     if (page_size == (1 << b)) page_shift = b;
@@ -336,19 +370,21 @@ static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void
   grid.x = static_cast<unsigned>((static_cast<int64_t>(n_tiles) * n_splits + per_group - 1) / per_group);
   hipLaunchKernelGGL((attn_mfma_kernel<NB, QT, PF, GQ>), grid, dim3(64 * per_group), 0, stream, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, positions, (__bf16*)out, part_o, part_ml,
-                     n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window, page_shift);
+                     n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window, page_shift, sink,
+                     reinterpret_cast<const float2*>(turn_back));
 }
 
 // Workspace (when n_splits > 1): part_o float32 [tokens * heads * n_splits * head_dim],
 // part_ml float32 [tokens * heads * n_splits * 2].
 // grouped: every tile is ONE token (tile_rows is not read), and a wavefront serves the query heads of one key/value
 // head together (at most 16 of them; tile_queries 16).
-extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
-                                 const int32_t* tile_seq, const int32_t* tile_q0, const int32_t* tile_rows,
-                                 const int32_t* positions, void* out, float* part_o, float* part_ml, int64_t tokens,
-                                 int n_tiles, int tile_queries, int n_splits, int heads, int kv_heads, int head_dim,
-                                 int page_size, int max_blocks, float scale, int window, int prefetch, int grouped,
-                                 hipStream_t stream) {
+static int attention_mfma_any(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                              const int32_t* tile_seq, const int32_t* tile_q0, const int32_t* tile_rows,
+                              const int32_t* positions, void* out, float* part_o, float* part_ml, int64_t tokens,
+                              int n_tiles, int tile_queries, int n_splits, int heads, int kv_heads, int head_dim,
+                              int page_size, int max_blocks, float scale, int window, int prefetch, int grouped,
+                              const float* sink, const float* turn_back, hipStream_t stream) {
+  IX_REQUIRE(turn_back == nullptr || head_dim % 32 == 0, "a result that is rotated back needs heads of a multiple of 32");
   IX_REQUIRE(tile_queries == 16 || tile_queries == 32, "a query tile holds up to 16 or 32 queries");
   IX_REQUIRE(tile_queries == 16 || head_dim <= 128, "tiles of 32 queries need head_dim <= 128");
   IX_REQUIRE(tokens >= 0 && n_tiles >= 0 && heads > 0 && kv_heads > 0 && max_blocks > 0, "sizes must be positive");
@@ -367,7 +403,7 @@ extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void*
   const float scale_log2 = scale * 1.4426950408889634f;
 #define ARGS                                                                                                    \
   grid, stream, q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, positions, out, part_o, part_ml, \
-      n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window
+      n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window, sink, turn_back
 #define CASE(NB)                                                    \
   case NB:                                                          \
     if (grouped) {                                                  \
@@ -394,8 +430,35 @@ extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void*
 #undef CASE4
 #undef ARGS
   if (ix_check_launch("ix_attention_mfma")) return 1;
-  if (n_splits > 1) return ix_attention_combine(part_o, part_ml, out, tokens, heads, n_splits, head_dim, stream);
+  if (n_splits > 1)
+    return ix_attention_combine(part_o, part_ml, out, tokens, heads, n_splits, head_dim, stream, turn_back);
   return 0;
+}
+
+extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                 const int32_t* tile_seq, const int32_t* tile_q0, const int32_t* tile_rows,
+                                 const int32_t* positions, void* out, float* part_o, float* part_ml, int64_t tokens,
+                                 int n_tiles, int tile_queries, int n_splits, int heads, int kv_heads, int head_dim,
+                                 int page_size, int max_blocks, float scale, int window, int prefetch, int grouped,
+                                 hipStream_t stream) {
+  return attention_mfma_any(q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, positions, out, part_o,
+                            part_ml, tokens, n_tiles, tile_queries, n_splits, heads, kv_heads, head_dim, page_size,
+                            max_blocks, scale, window, prefetch, grouped, nullptr, nullptr, stream);
+}
+
+// The same with a sink per head (float32 [heads], or null) in every softmax's denominator, and with the result of
+// every (token, head) rotated back by the token's angles (turn_back float32 (cos, sin) [tokens, head_dim / 2], or
+// null; head_dim a multiple of 32).
+extern "C" int ix_attention_mfma_sink(const void* q, const void* k_cache, const void* v_cache,
+                                      const int32_t* block_table, const int32_t* tile_seq, const int32_t* tile_q0,
+                                      const int32_t* tile_rows, const int32_t* positions, void* out, float* part_o,
+                                      float* part_ml, int64_t tokens, int n_tiles, int tile_queries, int n_splits,
+                                      int heads, int kv_heads, int head_dim, int page_size, int max_blocks, float scale,
+                                      int window, int prefetch, int grouped, const float* sink, const float* turn_back,
+                                      hipStream_t stream) {
+  return attention_mfma_any(q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, positions, out, part_o,
+                            part_ml, tokens, n_tiles, tile_queries, n_splits, heads, kv_heads, head_dim, page_size,
+                            max_blocks, scale, window, prefetch, grouped, sink, turn_back, stream);
 }
 
 // ---- the same operation without a workspace argument -----------------------------------------------------------

@@ -145,8 +145,9 @@ __device__ __forceinline__ float ix_glu(float g, float u, float limit) {
 #include <string>
 void ix_set_error(const std::string& msg);
 // out[t, h, :] from the parts that kernels which cut keys into slices leave (attention_mfma.hip)
+// (turn_back: float32 (cos, sin) [tokens, head_dim / 2]; the result is rotated by minus these angles, or null)
 int ix_attention_combine(const float* part_o, const float* part_ml, void* out, int64_t tokens, int heads,
-                         int n_splits, int head_dim, hipStream_t stream);
+                         int n_splits, int head_dim, hipStream_t stream, const float* turn_back = nullptr);
 int ix_check_launch(const char* what);
 #define IX_REQUIRE(cond, msg)                          \
   do {                                                 \

@@ -11,9 +11,10 @@
 //
 // As for the delta rule, the columns of S are independent, so the work is spread over (request, head, block of 16
 // value columns): a wavefront each, four lanes per column that own every fourth row (or, VEC, a quarter of the rows
-// side by side, read in 16-byte pieces).  Every lane also carries n for its rows and m (the same in all columns); the
-// first block of a head writes them back.  In the slot a head's matrix lies [column][row]; after the matrices of
-// all heads come n [heads][dim] and m [heads].
+// side by side, read in 16-byte pieces).  Every lane also carries n for its rows and m (the same in all columns).
+// Every block of columns keeps a copy of n and m of its own in the slot and reads and writes no other's: a block that
+// starts late must not find what an earlier one has already moved on.  In the slot a head's matrix lies
+// [column][row]; after the matrices of all heads come, per block of 16 columns, n [heads][dim] and m [heads].
 #include "common.h"
 
 typedef float mm_f32x4 __attribute__((ext_vector_type(4)));
@@ -58,8 +59,9 @@ matrix_memory_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* 
   const int cj = live ? col : vdim - 1;  // lanes past the last column repeat it and store nothing
   float* slot = state + static_cast<int64_t>(state_slots[seq]) * state_stride;
   float* sp = slot + static_cast<int64_t>(head) * dim * vdim;
-  float* np_ = slot + static_cast<int64_t>(heads) * dim * vdim + static_cast<int64_t>(head) * dim;
-  float* mp = slot + static_cast<int64_t>(heads) * dim * vdim + static_cast<int64_t>(heads) * dim + head;
+  float* mine = slot + static_cast<int64_t>(heads) * dim * vdim + static_cast<int64_t>(blockIdx.x) * (heads * dim + heads);
+  float* np_ = mine + static_cast<int64_t>(head) * dim;
+  float* mp = mine + static_cast<int64_t>(heads) * dim + head;
   const int quarter = dim / MM_SPLIT;
   auto row_of = [&](int r) { return VEC ? (r < quarter ? part * quarter + r : dim) : r * MM_SPLIT + part; };
   float S[RPL], N[RPL];
@@ -146,7 +148,7 @@ matrix_memory_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* 
       if (i < dim) sp[static_cast<int64_t>(col) * dim + i] = S[r];
     }
   }
-  if (blockIdx.x == 0 && lane < MM_SPLIT) {  // (every block of the head holds the same n and m)
+  if (lane < MM_SPLIT) {  // (the block's own copy of n and m)
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
       const int i = row_of(r);
@@ -158,14 +160,16 @@ matrix_memory_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* 
 
 // q, k [T, heads * dim] and v [T, heads * vdim] of the run's type with their row strides; gates float32 [T, 2 heads]
 // (the input gate's logits, then the forget gate's) and gate_bias float32 [2 heads] likewise; state: slot s at
-// state + s * state_stride, [heads, vdim, dim] then [heads, dim] then [heads]; out float32 [T, heads, vdim].
+// state + s * state_stride, [heads, vdim, dim], then per block of 16 value columns [heads, dim] and [heads]; out
+// float32 [T, heads, vdim].
 extern "C" int ix_matrix_memory(const void* q, const void* k, const void* v, int dtype, int64_t q_stride, int64_t k_stride,
                                 int64_t v_stride, const float* gates, const float* gate_bias, float cap, float* state,
                                 int64_t state_stride, const int32_t* q_start, const int32_t* state_slots, float* out,
                                 int64_t tokens, int requests, int heads, int dim, int vdim, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && requests >= 0 && heads > 0 && dim > 0 && vdim > 0 && cap > 0.f, "sizes must be positive");
   IX_REQUIRE(dim <= 256, "at most 256 numbers per query and key head");
-  IX_REQUIRE(state_stride >= static_cast<int64_t>(heads) * dim * vdim + static_cast<int64_t>(heads) * dim + heads,
+  IX_REQUIRE(state_stride >= static_cast<int64_t>(heads) * dim * vdim +
+                                 static_cast<int64_t>((vdim + MM_COLS - 1) / MM_COLS) * (heads * dim + heads),
              "state blocks too small");
   IX_REQUIRE(heads <= 65535 && requests <= 65535, "too many heads or requests for one launch");
   IX_REQUIRE(dtype == IX_F32 || dtype == IX_BF16, "dtype must be float32 or bfloat16");

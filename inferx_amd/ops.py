@@ -309,7 +309,8 @@ def rotate_heads(x: torch.Tensor, cos_sin: torch.Tensor, inverse: bool = False) 
 def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, n_splits: int,
                    workspace: Optional[torch.Tensor], scale: float, window: int, tile_queries: int = 16,
-                   prefetch: bool = False, grouped: bool = False) -> None:
+                   prefetch: bool = False, grouped: bool = False, sink: Optional[torch.Tensor] = None,
+                   turn_back: Optional[torch.Tensor] = None) -> None:
     """Paged attention on the matrix cores (bfloat16).  `tiles` int32 [3, n_tiles]: request, first token row and
     number of rows (<= tile_queries, which is 16 or 32) of each query tile.  `workspace` float32 with T * heads * n_splits * (d + 2) entries
     when n_splits > 1.  `grouped`: every tile is ONE token, and the query heads of a key/value head (at most 16)
@@ -334,11 +335,20 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
               f"workspace of {need} float32 needed")
         part_o = workspace
         part_ml = workspace[T * heads * n_splits * d:]
-    _call("ix_attention_mfma", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
-          _ptr(tiles[1]), _ptr(tiles[2]), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), _i64(T),
-          _i32(n_tiles), _i32(tile_queries), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(page_size),
-          _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(1 if prefetch else 0),
-          _i32(1 if grouped else 0), _stream())
+    args = (_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
+            _ptr(tiles[1]), _ptr(tiles[2]), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), _i64(T),
+            _i32(n_tiles), _i32(tile_queries), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(page_size),
+            _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(1 if prefetch else 0),
+            _i32(1 if grouped else 0))
+    if sink is None and turn_back is None:
+        _call("ix_attention_mfma", *args, _stream())
+        return
+    # `sink` float32 [heads]: exp(sink) joins every softmax's denominator; `turn_back` float32 [T, d / 2, 2]: the
+    # result of every (token, head) is rotated by minus these angles, halves paired (d a multiple of 32)
+    _need(sink is None or (sink.dtype == torch.float32 and sink.numel() == heads), "one float32 sink per head")
+    _need(turn_back is None or (turn_back.dtype == torch.float32 and turn_back.shape == (T, d // 2, 2) and d % 32 == 0
+                                and turn_back.is_contiguous()), "turn_back must be float32 [T, d / 2, 2], d a multiple of 32")
+    _call("ix_attention_mfma_sink", *args, _ptr(sink), _ptr(turn_back), _stream())
 
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -1133,11 +1143,17 @@ def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ab: torch.Tens
           _i32(dim), _i32(vdim), _stream())
 
 
+def matrix_memory_state_floats(heads: int, dim: int, vdim: int) -> int:
+    """Floats of a request's state for `matrix_memory`: the matrices, then n and m once per sixteen value columns."""
+    return heads * dim * vdim + -(-vdim // 16) * (heads * dim + heads)
+
+
 def matrix_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor,
                   cap: float, state: torch.Tensor, rows: StepRows, out: torch.Tensor, heads: int, dim: int,
                   vdim: int) -> None:
     """The matrix memory with exponential gates over the rows of a step, request by request, from and to `state` (a
-    float32 view [slots, >= heads * dim * vdim + heads * dim + heads]: matrices, then n, then the running maxima).
+    float32 view [slots, >= matrix_memory_state_floats(...)]: matrices, then per sixteen value columns n and the
+    running maxima).
     q, k [T, heads * dim], v [T, heads * vdim] (rows may be strided); gates float32 [T, 2 heads] (input gate's logits,
     then forget gate's), gate_bias float32 [2 heads]; out float32 [T, heads, vdim]."""
     T = q.shape[0]
@@ -1148,7 +1164,7 @@ def matrix_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torc
     _need(gate_bias.dtype == torch.float32 and gate_bias.numel() == 2 * heads and gate_bias.is_contiguous(),
           "gate_bias must be float32 [2 heads]")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
-          and state.shape[1] >= heads * dim * vdim + heads * dim + heads, "the state must be float32 [slots, >= matrices + n + m]")
+          and state.shape[1] >= matrix_memory_state_floats(heads, dim, vdim), "the state must be float32 [slots, >= matrices + n + m]")
     _need(out.dtype == torch.float32 and out.shape == (T, heads, vdim) and out.is_contiguous(), "out must be float32 [T, heads, vdim]")
     rows.check(T)
     S = rows.q_start.numel() - 1

@@ -165,11 +165,15 @@ class PagedAttention(Mixer):
         steps of one token per request); else the plain one, which also knows a sink, values of another size than
         keys and a result that is rotated back (`turn_back`: the table of the query's angles)."""
         page_size = cache.k.shape[2]
-        special = self.sink is not None or turn_back is not None or self.value_dim != self.head_dim
-        if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0 and not special:
+        # a sink and a result that is rotated back: the wavefront-level matrix-core kernel knows both (the latter for
+        # heads of a multiple of 32); values of another size than keys: the plain kernel
+        special = self.sink is not None or turn_back is not None
+        fits = self.value_dim == self.head_dim and (turn_back is None or self.head_dim % 32 == 0)
+        if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0 and fits:
             T = ctx.num_tokens
+            more = {"sink": self.sink, "turn_back": turn_back} if special else {}
             if not ctx.one_token_each:  # some request brings more than one token: the step's plan says who goes where
-                lds_fits = self.head_dim <= 128 and page_size & (page_size - 1) == 0
+                lds_fits = self.head_dim <= 128 and page_size & (page_size - 1) == 0 and not special
                 tile = WIDE_PREFILL_TILE if self.head_dim % 32 == 0 else PREFILL_TILE
                 lds, waves = mixed_step_plan(ctx, self.window, self.num_heads, self.num_kv_heads, lds_fits, tile)
                 table = ctx.block_tables[cache.group]
@@ -184,12 +188,14 @@ class PagedAttention(Mixer):
                     # a launch that serves some of the step's requests gets their rows put side by side
                     qs = q if rows is None else q.index_select(0, rows)
                     outs = out if rows is None else torch.empty_like(qs)
+                    if turn_back is not None:
+                        more["turn_back"] = turn_back if rows is None else turn_back.index_select(0, rows)
                     work = None
                     if n_splits > 1:
                         work = ctx.rt.empty((qs.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),),
                                             torch.float32)
                     ops.attention_mfma(qs, cache.k, cache.v, table, tiles, positions, outs, n_splits, work,
-                                       self.scale, self.window, QUERY_TILE, grouped=grouped)
+                                       self.scale, self.window, QUERY_TILE, grouped=grouped, **more)
                     if rows is not None:
                         out.index_copy_(0, rows, outs)
                 return
@@ -199,7 +205,7 @@ class PagedAttention(Mixer):
             if n_splits > 1:
                 work = ctx.rt.empty((q.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),), torch.float32)
             ops.attention_mfma(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, out,
-                               n_splits, work, self.scale, self.window, tile, prefetch=True, grouped=grouped)
+                               n_splits, work, self.scale, self.window, tile, prefetch=True, grouped=grouped, **more)
         else:
             ops.attention_plain(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.seq_of_token, ctx.positions,
                                 out, self.scale, self.window, self.sink, turn_back)

@@ -9,7 +9,8 @@ token scales, adds to and reads.
     y = (o / rms(o over the head) * norm_weight * sigmoid(gate)) . Wo^T   norm_weight of all heads' size
 
 State per request, float32, in the request's state slot: the heads' matrices (a column's rows side by side, as the
-kernel reads them), then n, then m; nothing is kept in pages.  Gates, maxima, exponentials, the recurrence and the
+kernel reads them), then n and m once per sixteen value columns (every block of the kernel carries its own copy, so
+that none reads what another has already moved on); nothing is kept in pages.  Gates, maxima, exponentials, the recurrence and the
 head norm are float32 in every run.
 """
 from __future__ import annotations
@@ -34,7 +35,7 @@ class MatrixMemoryMixer(Mixer):
         self.value_dim, self.gate_cap = int(value_dim), float(gate_cap)
         self.norm_eps, self.init_std = float(norm_eps), float(init_std)
         self.qk_dim, self.v_dim = self.num_heads * self.head_dim, self.num_heads * self.value_dim
-        self.state_floats = self.qk_dim * self.value_dim + self.qk_dim + self.num_heads
+        self.state_floats = ops.matrix_memory_state_floats(self.num_heads, self.head_dim, self.value_dim)
         self.w_in = self.w_gates = self.b_gates = self.w_out = self.norm_weight = None
 
     def param_specs(self) -> List[ParamSpec]:

@@ -127,9 +127,11 @@ def plain_sink_attention(q, keys, values, pos, scale, window, sink, angles):
     return out
 
 
-def run_sink_attention(paged, lengths, contexts, H, scale, window, sink, turn, dtype, standout=None, q_scale=1.0):
-    """The last lengths[i] positions of request i as one step's rows through `ops.attention_plain`; the kernel's
-    result and the float64 one.  standout = (request, key): the request's queries are made to match that key."""
+def run_sink_attention(paged, lengths, contexts, H, scale, window, sink, turn, dtype, standout=None, q_scale=1.0,
+                       mfma=False, splits=1, grouped=False):
+    """The last lengths[i] positions of request i as one step's rows through `ops.attention_plain` (or, `mfma`, the
+    wavefront-level matrix-core kernel in tiles of 16 queries, the keys in `splits` slices); the kernel's result and
+    the float64 one.  standout = (request, key): the request's queries are made to match that key."""
     from inferx_amd import ops
     G, d, vd = paged.keys[0].shape[1], paged.keys[0].shape[2], paged.values[0].shape[2]
     T = sum(lengths)
@@ -148,9 +150,20 @@ def run_sink_attention(paged, lengths, contexts, H, scale, window, sink, turn, d
         angles = torch.from_numpy(pos).double()[:, None] * freq[None, :]
         table = torch.stack([torch.cos(angles), torch.sin(angles)], dim=-1).float().contiguous().to(DEV)
     out = torch.empty(T, H, vd, dtype=dtype, device=DEV)
-    ops.attention_plain(q.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), torch.from_numpy(seq).to(DEV),
-                        torch.from_numpy(pos).to(DEV), out, scale, window, None if sink is None else sink.to(DEV),
-                        table if turn else None)
+    if mfma:
+        tiles, at = [], 0
+        for i, n in enumerate(lengths):
+            tiles += [(i, at + first, min(1 if grouped else 16, n - first)) for first in range(0, n, 1 if grouped else 16)]
+            at += n
+        tiles = torch.tensor(tiles, dtype=torch.int32).t().contiguous().to(DEV)
+        work = torch.empty(T * H * splits * (d + 2), dtype=torch.float32, device=DEV) if splits > 1 else None
+        ops.attention_mfma(q.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), tiles,
+                           torch.from_numpy(pos).to(DEV), out, splits, work, scale, window, 16, prefetch=splits > 1,
+                           grouped=grouped, sink=None if sink is None else sink.to(DEV), turn_back=table if turn else None)
+    else:
+        ops.attention_plain(q.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), torch.from_numpy(seq).to(DEV),
+                            torch.from_numpy(pos).to(DEV), out, scale, window, None if sink is None else sink.to(DEV),
+                            table if turn else None)
     want = torch.zeros(T, H, vd, dtype=F)
     for t in range(T):
         i = int(seq[t])
@@ -179,20 +192,43 @@ def test_attention_with_sink_window_and_values_turned_back(H, G, d, vd, page, wi
             assert float((got - want).abs().max()) <= tol * float(want.abs().max()), f"{lengths} sink {use_sink}"
 
 
+@pytest.mark.parametrize("H,G,d,page,window", [(4, 2, 32, 16, 9), (8, 1, 64, 16, 96), (16, 4, 128, 32, 40), (3, 3, 96, 16, 0),
+                                                (2, 1, 48, 48, 33)])
+def test_attention_with_sink_on_the_matrix_cores(H, G, d, page, window):
+    """The wavefront-level matrix-core kernel with a sink and the result turned back (heads of a multiple of 32; of 48:
+    the sink alone): portions in tiles of sixteen queries, single tokens with their keys in slices, single tokens with
+    the query heads of a key/value head side by side."""
+    contexts = [70, 33, 1, 150, 48]
+    sink = rnd((H,), 12, 1.5)
+    turn = d % 32 == 0
+    for lengths, splits, grouped in (([70, 20, 1, 9, 16], 1, False), ([1, 1, 1, 1, 1], 4, False), ([1, 1, 1, 1, 1], 2, H // G > 1),
+                                     ([3, 1, 1, 2, 1], 1, False)):
+        paged = PagedKV(contexts, G, d, d, page, torch.bfloat16, seed=3)
+        if window:
+            for i, (c, n) in enumerate(zip(contexts, lengths)):
+                paged.give_back(i, max(0, c - n + 1 - window))
+        for use_sink in (True, False):
+            got, want = run_sink_attention(paged, lengths, contexts, H, d ** -0.5, window, sink if use_sink else None,
+                                           turn, torch.bfloat16, mfma=True, splits=splits, grouped=grouped)
+            assert torch.isfinite(got).all()
+            assert float((got - want).abs().max()) <= 2e-2 * float(want.abs().max()), f"{lengths} {splits} sink {use_sink}"
+
+
+@pytest.mark.parametrize("mfma", [False, True])
 @pytest.mark.parametrize("window", [40, 96])
 @pytest.mark.parametrize("back", [0, 1, 15, 16, 17, "in", "out", "far"])
-def test_one_key_that_stands_out_at_the_windows_edge(window, back):
+def test_one_key_that_stands_out_at_the_windows_edge(window, back, mfma):
     """600 keys; the queries match ONE key strongly.  The key lies `back` places behind the last query: the query's own
     place, the one before, around a page's border, the last place inside the window ("in"), the first outside ("out") and
     far outside.  Inside, the result is that key's value (turned by the distance); outside, the key must not count."""
-    n, H, G, d, vd = 600, 4, 2, 32, 16
+    n, H, G, d, vd = 600, 4, 2, 32, (32 if mfma else 16)
     distance = {"in": window - 1, "out": window, "far": 400}.get(back, back)
     key = n - 1 - distance
     paged = PagedKV([n], G, d, vd, 16, torch.bfloat16, seed=21)
     sink = torch.full((H,), -2.0)
     for lengths in ([1], [24]):
         got, want = run_sink_attention(paged, lengths, [n], H, 0.25, window, sink, True, torch.bfloat16,
-                                       standout=(0, key), q_scale=0.2)
+                                       standout=(0, key), q_scale=0.2, mfma=mfma, splits=4 if mfma and lengths == [1] else 1)
         last_got, last_want = got[-1], want[-1]
         peak = float(paged.values[0][key].double().abs().max())
         if distance < window:  # nearly all the weight is on the key: the result has its value's size
@@ -421,7 +457,8 @@ def test_matrix_memory_over_steps_and_slots(H, d, vd, cap, dtype):
     from inferx_amd import ops
     steps = [(33, 16, 1), (1, 1, 1), (1, 1, 1), (2, 17, 5), (70, 1, 31)]
     slots = [4, 0, 2]
-    floats = H * d * vd + H * d + H
+    floats = ops.matrix_memory_state_floats(H, d, vd)
+    assert floats == H * d * vd + -(-vd // 16) * (H * d + H)
     state = torch.zeros(6, floats + 3, dtype=torch.float32, device=DEV)
     state[1] = float("nan")
     own = [(torch.zeros(H, d, vd, dtype=F), torch.zeros(H, d, dtype=F), torch.zeros(H, dtype=F)) for _ in slots]
@@ -444,9 +481,11 @@ def test_matrix_memory_over_steps_and_slots(H, d, vd, cap, dtype):
             at += length
     for i, slot in enumerate(slots):
         S = state[slot, :H * d * vd].view(H, vd, d).transpose(1, 2).cpu().double()
-        nvec = state[slot, H * d * vd:H * d * vd + H * d].view(H, d).cpu().double()
-        top = state[slot, H * d * vd + H * d:floats].cpu().double()
         assert float((S - own[i][0]).abs().max()) <= tol * max(float(own[i][0].abs().max()), 1e-3)
-        assert float((nvec - own[i][1]).abs().max()) <= tol * max(float(own[i][1].abs().max()), 1e-3)
-        assert float((top - own[i][2]).abs().max()) <= 1e-4 * max(float(own[i][2].abs().max()), 1.0)
+        for block in range(-(-vd // 16)):  # every block of sixteen columns carries n and m of its own
+            at = H * d * vd + block * (H * d + H)
+            nvec = state[slot, at:at + H * d].view(H, d).cpu().double()
+            top = state[slot, at + H * d:at + H * d + H].cpu().double()
+            assert float((nvec - own[i][1]).abs().max()) <= tol * max(float(own[i][1].abs().max()), 1e-3)
+            assert float((top - own[i][2]).abs().max()) <= 1e-4 * max(float(own[i][2].abs().max()), 1.0)
     assert torch.isnan(state[1]).all() and float(state[3].abs().max()) == 0.0

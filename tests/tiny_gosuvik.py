@@ -86,7 +86,7 @@ C = config(97, 40, 1e-5, 1, [
 D = config(256, 128, 1e-5, 4, [
     delta(2, 1, 64, 40, 4, experts(32, 8, 3)),
     latent(16, 24, 32, 40, 64, 0.15, 33, rot(32, 1000.0, yarn(6.0, 32, 16.0, 2.0)), dense(96)),
-    pair((8, 2, 32, 64, 0.2, 40, rot(32, 5000.0, {"factor": 2.0})), (2, 64, 32, 6.0), 0.8, 1.1, experts(32, 8, 2)),
+    pair((8, 2, 32, 32, 0.2, 40, rot(16, 5000.0, {"factor": 2.0})), (2, 64, 24, 6.0), 0.8, 1.1, experts(32, 8, 2)),
     delta(1, 1, 128, 32, 4, None),
     delta(4, 4, 32, 16, 2, dense(64)),
 ], loop=(1, 2, 2))
