@@ -35,6 +35,7 @@ feed-forward width, vocabulary and layers), both through the step function, at a
     python bench.py --workload pelalix [--sizes 2k,4k] [--layers L] [--batch B] [--prompt-len C] [--prefill-tokens N]
     python bench.py --workload dezudra [--sizes 1k,2k] [--layers L] [--batch B] [--prompt-len C] [--prefill-tokens N]
     python bench.py --workload bibevik [--sizes 1k,2k] [--only bibevik|dezudra]       # Bibevik beside Dezudra
+    python bench.py --workload gosuvik [--sizes 1k,2k] [--only gosuvik|dezudra]       # Gosuvik beside Dezudra
 
 and a whole batch through the engine's loop (scheduler, portions, decode graphs as they come, sampling) at the same
 shape:
@@ -632,6 +633,94 @@ def run_bibevik(args) -> int:
     return 0
 
 
+# Layer sizes for `--workload gosuvik`: width, attention heads and key/value heads of `dim` numbers (the latent layers:
+# per head `dim` plain and `rot` rotated query numbers, a latent of `rank`), the matrix memory's heads, windows,
+# experts, experts per token, an expert's width, the dense feed-forward's width, vocabulary
+GOSUVIK_SIZES = {
+    "1k": dict(width=1024, heads=8, kv_heads=2, dim=128, rot=64, rank=512, memory_heads=4, window=1024, experts=16,
+               top=4, ff=704, dense_ff=2816, vocab=32000),
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, rot=64, rank=512, memory_heads=8, window=1024, experts=32,
+               top=4, ff=1408, dense_ff=5632, vocab=32000),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, rot=64, rank=512, memory_heads=16, window=1024, experts=64,
+               top=8, ff=1408, dense_ff=11008, vocab=32000),
+}
+
+
+def run_gosuvik(args) -> int:
+    """Prefill of one prompt and decode steps of a batch, through the step function, for the Gosuvik design (layers
+    in turn: the delta rule with a decay per key channel, latent attention with a window and a gate, the pair of a
+    windowed attention with a sink and rotated values beside a matrix memory, latent attention again; norms in two
+    groups; experts chosen by a softmax router, the second layer's feed-forward dense with the PolyNorm activation)
+    and for the Dezudra design (the gated delta rule and differential attention with a window in turn, experts chosen
+    among groups) at equal width, attention heads, head size, window, experts and experts per token.  One JSON line;
+    per size and model milliseconds and tokens a second of both phases, and Gosuvik's time over the other's."""
+    import torch
+    from inferx_amd.config import config_from_dict
+    from inferx_amd.engine.runtime import Runtime
+
+    L = args.layers or 4
+    B, C, N = args.batch, args.prompt_len, args.prefill_tokens
+    rt = Runtime(args.dtype, "cuda:0")
+    gen = torch.Generator().manual_seed(1234)
+    out = {}
+
+    def specs(z):
+        H, G, D, W = z["heads"], z["kv_heads"], z["dim"], z["window"]
+        moe = {"kind": "moe", "expert": {"ff": z["ff"]}, "router": {"experts": z["experts"], "top": z["top"]}}
+        yarn = {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+        latent = lambda mlp: {"type": "latent_attention", "mlp": mlp,
+                              "mixer": {"heads": H, "dim": D, "rot_dim": z["rot"], "vdim": D, "kv_rank": z["rank"],
+                                        "scale": (D + z["rot"]) ** -0.5, "mask": {"size": W},
+                                        "rot": {"dims": z["rot"], "base": 10000.0, "scaling": yarn}}}
+        delta = {"type": "channel_delta", "mlp": moe,
+                 "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4, "decay_rank": 64, "gate_rank": 64}}
+        pair = {"type": "parallel", "mlp": moe,
+                "mixer": {"left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": W},
+                                   "rot": {"dims": D // 2, "base": 10000.0, "scaling": {"factor": 4.0}}},
+                          "right": {"heads": z["memory_heads"], "dim": D, "vdim": D, "gate_cap": 15.0},
+                          "left_scale": 0.5, "right_scale": 0.5}}
+        order = [delta, latent({"kind": "dense", "ff": z["dense_ff"]}), pair, latent(moe)]
+        gos = {"architecture": "Gosuvik", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6, "groups": 2},
+               "layers": [order[i % 4] for i in range(L)]}
+        dmlp = {"kind": "moe", "expert": {"ff": z["ff"]},
+                "router": {"experts": z["experts"], "top": z["top"], "groups": {"count": 4, "keep": 2}}}
+        ddelta = {"type": "delta", "mlp": dmlp, "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4}}
+        dattn = {"type": "attention", "mlp": dmlp,
+                 "mixer": {"heads": H, "kv_heads": G, "dim": D // 2, "vdim": D, "conv": 4, "scale": (D // 2) ** -0.5,
+                           "diff": 0.5, "rot": {"dims": D // 2, "base": 10000.0}, "mask": {"size": W, "keep_first": 4}}}
+        dez = {"architecture": "Dezudra", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+               "logit_scale": 1.0, "layers": [ddelta if i % 2 == 0 else dattn for i in range(L)]}
+        return {"gosuvik": config_from_dict(gos).model_spec(), "dezudra": config_from_dict(dez).model_spec()}
+
+    for name in [n for n in args.sizes.split(",") if n]:
+        z = GOSUVIK_SIZES[name]
+        res = {}
+        for which, spec in specs(z).items():
+            if args.only and which != args.only:
+                continue
+            log(f"{name}: {which}")
+            pre, dec = _time_prefill_and_decode(args, rt, spec, z["vocab"], gen)
+            res[which] = {"prefill_ms": round(pre * 1e3, 3), "prefill_tokens_s": round(N / pre, 1),
+                          "decode_ms": round(dec * 1e3, 3), "decode_tokens_s": round(B / dec, 1)}
+            log(f"{name}: {which}: {res[which]}")
+        if len(res) == 2:
+            res["gosuvik_over_dezudra"] = {
+                "prefill": round(res["gosuvik"]["prefill_ms"] / res["dezudra"]["prefill_ms"], 3),
+                "decode": round(res["gosuvik"]["decode_ms"] / res["dezudra"]["decode_ms"], 3)}
+        out[name] = dict(res, sizes=z)
+    first = out[next(iter(out))]
+    mine = first.get("gosuvik") or next(iter(v for v in first.values() if isinstance(v, dict) and "decode_ms" in v))
+    print(json.dumps({
+        "metric": f"Gosuvik decode tok/s @ batch {B} ({C}-token contexts), first size", "value": mine["decode_tokens_s"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": mine["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: seeded random weights and token ids",
+        "config": {"model": "Gosuvik beside Dezudra at equal sizes", "layers": L, "global_batch": B,
+                   "seq_len": C, "prefill_tokens": N, "parallelism": "single GPU", "page_size": PAGE},
+        "sizes": out}), flush=True)
+    return 0
+
+
 def run_pelalix(args) -> int:
     """Prefill of one prompt and decode steps of a batch, through the step function, for the Pelalix design and for
     the Qwen2-MoE architecture's dense layers (attention with rotation, RMS norms, the same gated feed-forward) at
@@ -714,7 +803,8 @@ def main() -> int:
                     help="fewer layers than the configuration has (sizes of a layer are never reduced)")
     ap.add_argument("--scarce", action="store_true", help="offline: so few pages that sequences are preempted")
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "mixed", "long", "mixed-small", "offline", "portion", "pelalix", "dezudra", "bibevik"],
+                    choices=["decode", "mixed", "long", "mixed-small", "offline", "portion", "pelalix", "dezudra", "bibevik",
+                             "gosuvik"],
                     help="decode, mixed-small: the Qwen1.5-MoE-A2.7B shape (decode is the default); mixed, long: the "
                          "Qwen2-57B-A14B shape")
     ap.add_argument("--batch", type=int, default=8)
@@ -726,8 +816,8 @@ def main() -> int:
     ap.add_argument("--prefill-context", type=int, default=0,
                     help="portion: tokens that the request has read before the timed portion")
     ap.add_argument("--shape", default="a27b", choices=["a27b", "57b"], help="portion: whose layer sizes")
-    ap.add_argument("--sizes", default="2k,4k", help="pelalix, dezudra, bibevik: which of the layer sizes " + ", ".join(PELALIX_SIZES))
-    ap.add_argument("--only", default="", help="bibevik: time one of the two models only (bibevik or dezudra)")
+    ap.add_argument("--sizes", default="2k,4k", help="pelalix, dezudra, bibevik, gosuvik: which of the layer sizes " + ", ".join(PELALIX_SIZES))
+    ap.add_argument("--only", default="", help="bibevik, gosuvik: time one of the two models only (by its name)")
     ap.add_argument("--prompt-len", type=int, default=PROMPT,
                     help="tokens of every request's prompt before it decodes (the context of the decode steps)")
     args = ap.parse_args()
@@ -735,9 +825,9 @@ def main() -> int:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
         return 2
     if args.steps is None:
-        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0, "portion": 2, "pelalix": 32, "dezudra": 32, "bibevik": 32}[args.workload]
+        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0, "portion": 2, "pelalix": 32, "dezudra": 32, "bibevik": 32, "gosuvik": 32}[args.workload]
     if args.warmup is None:
-        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0, "portion": 1, "pelalix": 4, "dezudra": 4, "bibevik": 4}[args.workload]
+        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0, "portion": 1, "pelalix": 4, "dezudra": 4, "bibevik": 4, "gosuvik": 4}[args.workload]
     if args.workload == "offline":
         return run_offline(args)
     if args.workload == "portion":
@@ -748,6 +838,8 @@ def main() -> int:
         return run_dezudra(args)
     if args.workload == "bibevik":
         return run_bibevik(args)
+    if args.workload == "gosuvik":
+        return run_gosuvik(args)
     if args.workload != "decode":
         return run_57b(args)
     if args.layers is None:

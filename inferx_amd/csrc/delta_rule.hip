@@ -7,9 +7,10 @@
 // size come from two small projections a, b (float32):  g = exp(-exp(A_log) softplus(a + dt_bias)),  beta =
 // sigmoid(b).  Everything but the loads of q, k, v is float32.
 //
-// A decay per key channel (`ach` given): g is a vector over the rows of S, g_i = exp(-exp(A_log) softplus(a_i +
-// dt_bias_i)) with a float32 [T, heads * dim] and dt_bias [heads * dim], S <- diag(g) S; `ab` then holds the step
-// size's logits alone, float32 [T, heads].
+// A decay per key channel (`ach` given): g is a vector over the rows of S, S <- diag(g) S, and `ach` float32
+// [T, heads * dim] holds the decays themselves, g_i = exp(-exp(A_log) softplus(a_i + dt_bias_i)), made once per token
+// and channel by ix_channel_decays (every block of a head's columns needs them all); `ab` then holds the step size's
+// logits alone, float32 [T, heads], and a_log and dt_bias are not read.
 //
 // The columns of S are independent recurrences (column j only ever meets v[j]), so the work is spread over
 // (request, head, block of 16 value columns): one wavefront each, four lanes per column that own every fourth row
@@ -84,19 +85,11 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
       S[r] = i < dim ? sp[static_cast<int64_t>(cj) * dim + i] : 0.f;
     }
   }
-  const float rate = expf(a_log[head]), bias = CH ? 0.f : dt_bias[head];
+  const float rate = CH ? 0.f : expf(a_log[head]), bias = CH ? 0.f : dt_bias[head];
   const float q_scale = 1.0f / sqrtf(static_cast<float>(dim));
-  float biasr[CH ? RPL : 1];  // a decay per key channel: the bias of each of this lane's rows
-  if constexpr (CH) {
-#pragma unroll
-    for (int r = 0; r < RPL; ++r) {
-      const int i = row_of(r);
-      biasr[r] = i < dim ? dt_bias[head * dim + i] : 0.f;
-    }
-  }
 
   float kc[RPL], qc[RPL], vc, ac, bc;  // the present row's operands
-  float gc[CH ? RPL : 1];               // (and the decay's logits of this lane's rows)
+  float gc[CH ? RPL : 1];               // (and the decays of this lane's rows)
   auto fetch = [&](int64_t row, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& aa, float& bb,
                    float (&gg)[CH ? RPL : 1]) {
     const T* qr = q + row * q_stride + kv * dim;
@@ -179,12 +172,8 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
     float dot = 0.f;
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
-      if constexpr (CH) {
-        const float xr = gc[r] + biasr[r];
-        S[r] *= expf(-rate * (xr > 20.f ? xr : log1pf(expf(xr))));
-      } else {
-        S[r] *= g;
-      }
+      if constexpr (CH) S[r] *= gc[r];
+      else S[r] *= g;
       dot += S[r] * (kc[r] * k_inv);
     }
     dot += ix_dpp<IX_DPP_XOR1>(dot);
@@ -282,11 +271,8 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
   float S[RPL];
 #pragma unroll
   for (int r = 0; r < RPL; ++r) S[r] = sp[static_cast<int64_t>(cj) * DIM + part * RPL + r];
-  const float rate = expf(a_log[head]), bias = CH ? 0.f : dt_bias[head];
+  const float rate = CH ? 0.f : expf(a_log[head]), bias = CH ? 0.f : dt_bias[head];
   const float q_scale = 1.0f / sqrtf(static_cast<float>(DIM));
-  // (piece u * 64 + lane of a chunk's decays is piece lane % G4 of a row whatever u: the bias is the lane's own)
-  delta_f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
-  if constexpr (CH) bias4 = *reinterpret_cast<const delta_f32x4*>(dt_bias + head * DIM + 4 * (lane % G4));
 
   delta_u32x4 st_qk[PER_LANE];
   delta_f32x4 st_g[G_PER_LANE];
@@ -354,13 +340,7 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
 #pragma unroll
       for (int u = 0; u < G_PER_LANE; ++u) {
         const int id = u * 64 + lane;
-        delta_f32x4 g;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float x = st_g[u][e] + bias4[e];
-          g[e] = expf(-rate * (x > 20.f ? x : log1pf(expf(x))));
-        }
-        g_s[id / G4][id % G4] = g;
+        g_s[id / G4][id % G4] = st_g[u];
       }
     }
   };
@@ -435,8 +415,8 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
 }
 
 // q, k [T, kv_heads * dim] and v [T, heads * vdim] of the run's type with their row strides; ab float32 [T, 2 heads]
-// (a then b); a_log, dt_bias float32 [heads]; or, with a decay per key channel, ach float32 [T, heads * dim], ab
-// float32 [T, heads] (b alone) and dt_bias float32 [heads * dim]; state: slot s at state + s * state_stride, [heads, vdim, dim] (a column's rows side by side);
+// (a then b); a_log, dt_bias float32 [heads]; or, with a decay per key channel, ach float32 [T, heads * dim] (the
+// decays themselves) and ab float32 [T, heads] (b alone); state: slot s at state + s * state_stride, [heads, vdim, dim] (a column's rows side by side);
 // out float32 [T, heads, vdim].
 extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dtype, int64_t q_stride,
                              int64_t k_stride, int64_t v_stride, const float* ab, const float* ach, const float* a_log,
@@ -457,7 +437,7 @@ extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dt
   const bool vec = dtype == IX_BF16 && dim % (8 * DELTA_SPLIT) == 0 && (q_stride * elt) % 16 == 0 && (k_stride * elt) % 16 == 0 &&
                    state_stride % 4 == 0 &&
                    ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(state) |
-                     reinterpret_cast<uintptr_t>(ach) | reinterpret_cast<uintptr_t>(dt_bias)) & 15) == 0;
+                     reinterpret_cast<uintptr_t>(ach)) & 15) == 0;
 #define LAUNCH_CH(TT, RPL, VEC, CH)                                                                                         \
   hipLaunchKernelGGL((delta_rule_kernel<TT, RPL, VEC, CH>), grid, block, 0, stream, (const TT*)q, (const TT*)k, (const TT*)v, \
                      q_stride, k_stride, v_stride, ab, ach, a_log, dt_bias, state, state_stride, q_start, state_slots, out,   \
@@ -498,10 +478,35 @@ extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dt
   return ix_check_launch("ix_delta_rule");
 }
 
+// x[t, h, i] <- exp(-exp(a_log[h]) softplus(x[t, h, i] + dt_bias[h, i])) in place: the decays per key channel
+// from their logits, float32 [T, heads * dim].
+__global__ void channel_decays_kernel(float* __restrict__ x, const float* __restrict__ a_log,
+                                      const float* __restrict__ dt_bias, int64_t n, int heads, int dim) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int c = static_cast<int>(i % (static_cast<int64_t>(heads) * dim));
+    const float v = x[i] + dt_bias[c];
+    x[i] = expf(-expf(a_log[c / dim]) * (v > 20.f ? v : log1pf(expf(v))));
+  }
+}
+
+extern "C" int ix_channel_decays(float* x, const float* a_log, const float* dt_bias, int64_t tokens, int heads, int dim,
+                                 hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && heads > 0 && dim > 0, "sizes must be positive");
+  if (tokens == 0) return 0;
+  const int64_t n = tokens * heads * dim;
+  hipLaunchKernelGGL(channel_decays_kernel, dim3(static_cast<unsigned>(std::min<int64_t>((n + 255) / 256, 65536))), dim3(256), 0,
+                     stream, x, a_log, dt_bias, n, heads, dim);
+  return ix_check_launch("ix_channel_decays");
+}
+
 // ---------------------------------------------------------------------------
 // What follows a mixer whose heads are normalised one by one, a wavefront per (token, head):
 //
 //   o = x - lambda x2  (x2 optional);  y = o / sqrt(mean(o^2) + eps) * weight (optional) * silu(gate) (optional) * mult
+//
+// With `den_a` (float32, one number per (token, head)) x is first divided by max(|den_a|, den_b) + 1e-6, den_b the
+// number at den_b[(t * heads + head) * den_b_stride] (a read-out that is normalised by its own size).
 //
 // x, x2 float32 [T, heads, vdim]; weight [vdim], shared by the heads (or [heads, vdim] with `weight_per_head`);
 // `gate_sigmoid`: sigmoid(gate) instead of silu(gate); gate of the run's type at
@@ -511,7 +516,8 @@ __global__ void __launch_bounds__(256)
 head_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ x2, float lambda,
                       const void* __restrict__ weight, int w_dtype, const T* __restrict__ gate, int64_t gate_stride,
                       T* __restrict__ out, int64_t pairs, int heads, int vdim, float eps, float mult,
-                      int weight_per_head, int gate_sigmoid) {
+                      int weight_per_head, int gate_sigmoid, const float* __restrict__ den_a,
+                      const float* __restrict__ den_b, int den_b_stride) {
   const int64_t p = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (p >= pairs) return;
   const int lane = threadIdx.x & 63;
@@ -519,13 +525,14 @@ head_norm_gate_kernel(const float* __restrict__ x, const float* __restrict__ x2,
   const int head = static_cast<int>(p % heads);
   const float* xr = x + p * vdim;
   const float* x2r = x2 ? x2 + p * vdim : nullptr;
+  const float pre = den_a ? 1.0f / (fmaxf(fabsf(den_a[p]), den_b[p * den_b_stride]) + 1e-6f) : 1.0f;
   float ss = 0.f;
   for (int j = lane; j < vdim; j += 64) {
-    const float o = x2r ? xr[j] - lambda * x2r[j] : xr[j];
+    const float o = (x2r ? xr[j] - lambda * x2r[j] : xr[j]) * pre;
     ss += o * o;
   }
   ss = ix_wave_sum(ss);
-  const float inv = mult / sqrtf(ss / static_cast<float>(vdim) + eps);
+  const float inv = pre * mult / sqrtf(ss / static_cast<float>(vdim) + eps);
   for (int j = lane; j < vdim; j += 64) {
     float y = (x2r ? xr[j] - lambda * x2r[j] : xr[j]) * inv;
     if (weight) y *= ix_load_rt(weight, w_dtype, weight_per_head ? head * vdim + j : j);
@@ -544,20 +551,22 @@ __global__ void __launch_bounds__(256)
 head_norm_gate_wide_kernel(const float* __restrict__ x, const float* __restrict__ x2, float lambda,
                            const void* __restrict__ weight, int w_dtype, const T* __restrict__ gate,
                            int64_t gate_stride, T* __restrict__ out, int heads, int vdim, float eps, float mult,
-                           int weight_per_head, int gate_sigmoid) {
+                           int weight_per_head, int gate_sigmoid, const float* __restrict__ den_a,
+                           const float* __restrict__ den_b, int den_b_stride) {
   __shared__ float red[16];
   const int64_t p = blockIdx.x;
   const int64_t t = p / heads;
   const int head = static_cast<int>(p % heads);
   const float* xr = x + p * vdim;
   const float* x2r = x2 ? x2 + p * vdim : nullptr;
+  const float pre = den_a ? 1.0f / (fmaxf(fabsf(den_a[p]), den_b[p * den_b_stride]) + 1e-6f) : 1.0f;
   float ss = 0.f;
   for (int j = threadIdx.x; j < vdim; j += 256) {
-    const float o = x2r ? xr[j] - lambda * x2r[j] : xr[j];
+    const float o = (x2r ? xr[j] - lambda * x2r[j] : xr[j]) * pre;
     ss += o * o;
   }
   ss = ix_block_sum(ss, red);
-  const float inv = mult / sqrtf(ss / static_cast<float>(vdim) + eps);
+  const float inv = pre * mult / sqrtf(ss / static_cast<float>(vdim) + eps);
   for (int j = threadIdx.x; j < vdim; j += 256) {
     float y = (x2r ? xr[j] - lambda * x2r[j] : xr[j]) * inv;
     if (weight) y *= ix_load_rt(weight, w_dtype, weight_per_head ? head * vdim + j : j);
@@ -572,8 +581,9 @@ head_norm_gate_wide_kernel(const float* __restrict__ x, const float* __restrict_
 extern "C" int ix_head_norm_gate(const float* x, const float* x2, float lambda, const void* weight, int w_dtype,
                                  const void* gate, int64_t gate_stride, void* out, int dtype, int64_t tokens,
                                  int heads, int vdim, float eps, float mult, int weight_per_head, int gate_sigmoid,
-                                 hipStream_t stream) {
+                                 const float* den_a, const float* den_b, int den_b_stride, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && heads > 0 && vdim > 0, "sizes must be positive");
+  IX_REQUIRE(den_a == nullptr || (den_b != nullptr && den_b_stride > 0), "a divisor comes as two numbers per row");
   IX_REQUIRE(dtype == IX_F32 || dtype == IX_BF16, "dtype must be float32 or bfloat16");
   if (tokens == 0) return 0;
   const int64_t pairs = tokens * heads;
@@ -584,21 +594,21 @@ extern "C" int ix_head_norm_gate(const float* x, const float* x2, float lambda, 
     if (dtype == IX_F32)
       hipLaunchKernelGGL(head_norm_gate_wide_kernel<float>, wide, threads, 0, stream, x, x2, lambda, weight, w_dtype,
                          (const float*)gate, gate_stride, (float*)out, heads, vdim, eps, mult, weight_per_head,
-                         gate_sigmoid);
+                         gate_sigmoid, den_a, den_b, den_b_stride);
     else
       hipLaunchKernelGGL(head_norm_gate_wide_kernel<bf16_t>, wide, threads, 0, stream, x, x2, lambda, weight, w_dtype,
                          (const bf16_t*)gate, gate_stride, (bf16_t*)out, heads, vdim, eps, mult, weight_per_head,
-                         gate_sigmoid);
+                         gate_sigmoid, den_a, den_b, den_b_stride);
     return ix_check_launch("ix_head_norm_gate");
   }
   dim3 grid(static_cast<unsigned>((pairs + 3) / 4)), block(256);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, x, x2, lambda, weight, w_dtype,
                        (const float*)gate, gate_stride, (float*)out, pairs, heads, vdim, eps, mult, weight_per_head,
-                       gate_sigmoid);
+                       gate_sigmoid, den_a, den_b, den_b_stride);
   else
     hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, stream, x, x2, lambda, weight, w_dtype,
                        (const bf16_t*)gate, gate_stride, (bf16_t*)out, pairs, heads, vdim, eps, mult, weight_per_head,
-                       gate_sigmoid);
+                       gate_sigmoid, den_a, den_b, den_b_stride);
   return ix_check_launch("ix_head_norm_gate");
 }

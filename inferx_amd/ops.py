@@ -1113,14 +1113,14 @@ def short_conv(x: torch.Tensor, bias: Optional[torch.Tensor], weight: torch.Tens
 
 def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor,
                dt_bias: torch.Tensor, state: torch.Tensor, rows: StepRows, out: torch.Tensor, heads: int,
-               kv_heads: int, dim: int, vdim: int, channel_logits: Optional[torch.Tensor] = None) -> None:
+               kv_heads: int, dim: int, vdim: int, channel_decays: Optional[torch.Tensor] = None) -> None:
     """The gated delta rule over the rows of a step, request by request, from and to `state` (a float32 view
     [slots, >= heads * dim * vdim]).  q, k [T, kv_heads * dim], v [T, heads * vdim] (rows may be strided);
     ab float32 [T, 2 heads]: the decay's and the step size's logits; out float32 [T, heads, vdim].
-    `channel_logits` float32 [T, heads * dim]: a decay per key channel from these logits, with dt_bias
-    [heads * dim]; ab is then float32 [T, heads], the step size's logits alone."""
+    `channel_decays` float32 [T, heads * dim]: a decay per key channel (the decays themselves, see
+    `channel_decays`); ab is then float32 [T, heads], the step size's logits alone, and dt_bias is not read."""
     T = q.shape[0]
-    per = 1 if channel_logits is None else dim
+    channel_logits = channel_decays
     for t, n in ((q, kv_heads * dim), (k, kv_heads * dim), (v, heads * vdim)):
         _need(t.dim() == 2 and t.shape == (T, n) and t.stride(1) == 1 and t.dtype == q.dtype and t.is_cuda, "q, k or v shape")
     if channel_logits is None:
@@ -1128,10 +1128,10 @@ def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ab: torch.Tens
     else:
         _need(ab.dtype == torch.float32 and ab.shape == (T, heads) and ab.is_contiguous(), "ab must be float32 [T, heads]")
         _need(channel_logits.dtype == torch.float32 and channel_logits.shape == (T, heads * dim)
-              and channel_logits.is_contiguous(), "the decays' logits must be float32 [T, heads * dim]")
+              and channel_logits.is_contiguous(), "the decays must be float32 [T, heads * dim]")
     _need(a_log.dtype == torch.float32 and a_log.numel() == heads and dt_bias.dtype == torch.float32
-          and dt_bias.numel() == heads * per and dt_bias.is_contiguous(),
-          "a_log must be float32 [heads], dt_bias float32 with one number per decay")
+          and (channel_logits is not None or dt_bias.numel() == heads) and dt_bias.is_contiguous(),
+          "a_log and dt_bias must be float32 [heads]")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
           and state.shape[1] >= heads * dim * vdim, "the state must be float32 [slots, >= heads * dim * vdim]")
     _need(out.dtype == torch.float32 and out.shape == (T, heads, vdim), "out must be float32 [T, heads, vdim]")
@@ -1143,19 +1143,30 @@ def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ab: torch.Tens
           _i32(dim), _i32(vdim), _stream())
 
 
+def channel_decays(logits: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, heads: int, dim: int) -> None:
+    """logits float32 [T, heads * dim] in place: exp(-exp(a_log[h]) softplus(logit + dt_bias[h, i])), the decay of
+    every head's every key channel."""
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[1] == heads * dim and logits.is_contiguous(),
+          "the logits must be float32 [T, heads * dim]")
+    _need(a_log.dtype == torch.float32 and a_log.numel() == heads and dt_bias.dtype == torch.float32
+          and dt_bias.numel() == heads * dim and dt_bias.is_contiguous(), "a_log float32 [heads], dt_bias float32 [heads * dim]")
+    _call("ix_channel_decays", _ptr(logits), _ptr(a_log), _ptr(dt_bias), _i64(logits.shape[0]), _i32(heads), _i32(dim), _stream())
+
+
 def matrix_memory_state_floats(heads: int, dim: int, vdim: int) -> int:
-    """Floats of a request's state for `matrix_memory`: the matrices, then n and m once per sixteen value columns."""
-    return heads * dim * vdim + -(-vdim // 16) * (heads * dim + heads)
+    """Floats of a request's state for `matrix_memory`: the matrices with n as one more column, then the maxima."""
+    return heads * dim * (vdim + 1) + heads
 
 
 def matrix_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor,
-                  cap: float, state: torch.Tensor, rows: StepRows, out: torch.Tensor, heads: int, dim: int,
-                  vdim: int) -> None:
+                  cap: float, state: torch.Tensor, rows: StepRows, out: torch.Tensor, nq: torch.Tensor,
+                  work: torch.Tensor, heads: int, dim: int, vdim: int) -> None:
     """The matrix memory with exponential gates over the rows of a step, request by request, from and to `state` (a
-    float32 view [slots, >= matrix_memory_state_floats(...)]: matrices, then per sixteen value columns n and the
-    running maxima).
-    q, k [T, heads * dim], v [T, heads * vdim] (rows may be strided); gates float32 [T, 2 heads] (input gate's logits,
-    then forget gate's), gate_bias float32 [2 heads]; out float32 [T, heads, vdim]."""
+    float32 view [slots, >= matrix_memory_state_floats(...)]: per head [vdim + 1, dim] with n as the last column, then
+    the running maxima).  q, k [T, heads * dim], v [T, heads * vdim] (rows may be strided); gates float32 [T, 2 heads]
+    (input gate's logits, then forget gate's), gate_bias float32 [2 heads].  Leaves out float32 [T, heads, vdim] =
+    S^T q', nq float32 [T, heads] = n . q' and work float32 [T, heads, 3] = (keep, take, exp(-m')): the read-out is
+    out / (max(|nq|, work[..., 2]) + 1e-6), which `head_norm_gate` forms on its way (`den_a`, `den_b`)."""
     T = q.shape[0]
     for t, n in ((q, heads * dim), (k, heads * dim), (v, heads * vdim)):
         _need(t.dim() == 2 and t.shape == (T, n) and t.stride(1) == 1 and t.dtype == q.dtype and t.is_cuda, "q, k or v shape")
@@ -1164,24 +1175,34 @@ def matrix_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torc
     _need(gate_bias.dtype == torch.float32 and gate_bias.numel() == 2 * heads and gate_bias.is_contiguous(),
           "gate_bias must be float32 [2 heads]")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
-          and state.shape[1] >= matrix_memory_state_floats(heads, dim, vdim), "the state must be float32 [slots, >= matrices + n + m]")
+          and state.shape[1] >= matrix_memory_state_floats(heads, dim, vdim), "the state must be float32 [slots, >= matrices + maxima]")
     _need(out.dtype == torch.float32 and out.shape == (T, heads, vdim) and out.is_contiguous(), "out must be float32 [T, heads, vdim]")
+    _need(nq.dtype == torch.float32 and nq.shape == (T, heads) and nq.is_contiguous(), "nq must be float32 [T, heads]")
+    _need(work.dtype == torch.float32 and work.shape == (T, heads, 3) and work.is_contiguous(), "work must be float32 [T, heads, 3]")
     rows.check(T)
     S = rows.q_start.numel() - 1
     _call("ix_matrix_memory", q.data_ptr(), k.data_ptr(), v.data_ptr(), _i32(_dt(q)), _i64(q.stride(0)), _i64(k.stride(0)),
           _i64(v.stride(0)), _ptr(gates), _ptr(gate_bias), _f32(cap), state.data_ptr(), _i64(state.stride(0)),
-          _ptr(rows.q_start), _ptr(rows.state_slots), _ptr(out), _i64(T), _i32(S), _i32(heads), _i32(dim), _i32(vdim),
-          _stream())
+          _ptr(rows.q_start), _ptr(rows.state_slots), _ptr(work), _ptr(out), _ptr(nq), _i64(T), _i32(S), _i32(heads),
+          _i32(dim), _i32(vdim), _stream())
 
 
 def head_norm_gate(x: torch.Tensor, out: torch.Tensor, eps: float, weight: Optional[torch.Tensor] = None,
                    gate: Optional[torch.Tensor] = None, x2: Optional[torch.Tensor] = None, lam: float = 0.0,
-                   mult: float = 1.0, weight_per_head: bool = False, gate_sigmoid: bool = False) -> None:
+                   mult: float = 1.0, weight_per_head: bool = False, gate_sigmoid: bool = False,
+                   den_a: Optional[torch.Tensor] = None, den_b: Optional[torch.Tensor] = None) -> None:
     """Per (token, head): o = x - lam * x2 (x2 optional); out = o / sqrt(mean(o^2) + eps) * weight * silu(gate) * mult.
     x, x2 float32 [T, heads, vdim]; weight [vdim] (`weight_per_head`: [heads, vdim]); `gate_sigmoid`: sigmoid(gate)
     instead of silu(gate); gate [T, >= heads * vdim] (rows may be strided) and out
-    [T, heads * vdim] of the run's type."""
+    [T, heads * vdim] of the run's type.  `den_a` float32 [T, heads] with `den_b` float32 [T, heads] (a view with any
+    stride between its numbers): x is first divided by max(|den_a|, den_b) + 1e-6."""
     T, heads, vdim = x.shape
+    stride_b = 0
+    if den_a is not None:
+        _need(den_a.dtype == torch.float32 and den_a.shape == (T, heads) and den_a.is_contiguous(), "den_a must be float32 [T, heads]")
+        _need(den_b is not None and den_b.dtype == torch.float32 and den_b.shape == (T, heads) and den_b.is_cuda
+              and (T == 0 or den_b.stride(0) == heads * den_b.stride(1)), "den_b must be float32 [T, heads], evenly strided")
+        stride_b = den_b.stride(1)
     _need(x.dtype == torch.float32 and (x2 is None or (x2.dtype == torch.float32 and x2.shape == x.shape)), "x, x2 float32")
     _need(out.shape == (T, heads * vdim), "out must be [T, heads * vdim]")
     _need(weight is None or weight.numel() == (heads * vdim if weight_per_head else vdim),
@@ -1193,7 +1214,8 @@ def head_norm_gate(x: torch.Tensor, out: torch.Tensor, eps: float, weight: Optio
         stride = gate.stride(0)
     _call("ix_head_norm_gate", _ptr(x), _ptr(x2), _f32(lam), _ptr(weight), _i32(_dt(weight) if weight is not None else F32),
           gate.data_ptr() if gate is not None else None, _i64(stride), _ptr(out), _i32(_dt(out)), _i64(T), _i32(heads),
-          _i32(vdim), _f32(eps), _f32(mult), _i32(1 if weight_per_head else 0), _i32(1 if gate_sigmoid else 0), _stream())
+          _i32(vdim), _f32(eps), _f32(mult), _i32(1 if weight_per_head else 0), _i32(1 if gate_sigmoid else 0),
+          _ptr(den_a), den_b.data_ptr() if den_a is not None else None, _i32(stride_b), _stream())
 
 
 def attention_diff_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,

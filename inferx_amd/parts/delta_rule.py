@@ -104,6 +104,7 @@ class GatedDeltaMixer(Mixer):
         if self.decay_rank:  # a decay per key channel: its logits through the second product, float32
             inner = proj[:, at + gate_width:at + gate_width + self.decay_rank].contiguous()
             channel_logits = rt.linear_f32(inner, self.w_a2)
+            ops.channel_decays(channel_logits, self.a_log, self.dt_bias, self.num_heads, self.head_dim)  # in place
         q, k, v = rt.empty((T, self.qk_dim)), rt.empty((T, self.qk_dim)), rt.empty((T, self.v_dim))
         matrices, tail = cache.state[:, :self.matrix_floats], cache.state[:, self.matrix_floats:]
         self.conv.apply(ctx, proj, tail, q, k, v, silu=True)

@@ -9,8 +9,9 @@ token scales, adds to and reads.
     y = (o / rms(o over the head) * norm_weight * sigmoid(gate)) . Wo^T   norm_weight of all heads' size
 
 State per request, float32, in the request's state slot: the heads' matrices (a column's rows side by side, as the
-kernel reads them), then n and m once per sixteen value columns (every block of the kernel carries its own copy, so
-that none reads what another has already moved on); nothing is kept in pages.  Gates, maxima, exponentials, the recurrence and the
+kernels read them) with n as one more column (its value is always 1), then the maxima; nothing is kept in pages.
+The chain of maxima runs first, in a launch of its own, so that the recurrence's blocks share nothing; the division
+rides on the kernel that normalises the heads.  Gates, maxima, exponentials, the recurrence and the
 head norm are float32 in every run.
 """
 from __future__ import annotations
@@ -62,13 +63,14 @@ class MatrixMemoryMixer(Mixer):
         gates = rt.linear_f32(x, self.w_gates)    # the two gates' logits, float32
         Q, V = self.qk_dim, self.v_dim
         q, k, v, gate = proj[:, :Q], proj[:, Q:2 * Q], proj[:, 2 * Q:2 * Q + V], proj[:, 2 * Q + V:]
-        o = rt.empty((T, H, self.value_dim), torch.float32)
+        o, nq = rt.empty((T, H, self.value_dim), torch.float32), rt.empty((T, H), torch.float32)
+        work = rt.empty((T, H, 3), torch.float32)  # keep, take, exp(-m') per token and head
         ops.matrix_memory(q, k, v, gates, self.b_gates, self.gate_cap, cache.state,
-                          ops.StepRows(ctx.seq_of_token, ctx.q_start, ctx.state_slots), o, H, self.head_dim,
+                          ops.StepRows(ctx.seq_of_token, ctx.q_start, ctx.state_slots), o, nq, work, H, self.head_dim,
                           self.value_dim)
         y = rt.empty((T, V))
         ops.head_norm_gate(o, y, self.norm_eps, weight=self.norm_weight, gate=gate, weight_per_head=True,
-                           gate_sigmoid=True)
+                           gate_sigmoid=True, den_a=nq, den_b=work[:, :, 2])
         return rt.linear(y, self.w_out)
 
 

@@ -83,7 +83,7 @@ def test_tensor_names_and_what_keeps_what():
     need, state = plan[4][0]["mixer"]
     assert need.window == 9 and [(a.name, a.heads, a.width, a.transposed) for a in need.arrays] == [("k", 2, 16, False), ("v", 2, 24, True)]
     need, state = plan[4][0]["second_mixer"]
-    assert need is None and state.shape == (2 * 12 * 20 + 2 * (2 * 12 + 2),)  # n and m once per sixteen columns
+    assert need is None and state.shape == (2 * 12 * (20 + 1) + 2,)  # n is one more column; then the maxima
     assert model.graph_safe()
 
 

@@ -394,8 +394,10 @@ def test_channel_delta_over_steps_and_slots(H, G, d, vd, dtype):
         q, k = rnd((T, G * d), 100 + n, 1.0, dtype), rnd((T, G * d), 200 + n, 1.0, dtype)
         v, b, a = rnd((T, H * vd), 300 + n, 1.0, dtype), rnd((T, H), 400 + n, 1.0), rnd((T, H * d), 500 + n, 1.5)
         out = torch.empty(T, H, vd, dtype=torch.float32, device=DEV)
+        decays = a.to(DEV)
+        ops.channel_decays(decays, a_log.to(DEV), dt_bias.to(DEV), H, d)
         ops.delta_rule(q.to(DEV), k.to(DEV), v.to(DEV), b.to(DEV), a_log.to(DEV), dt_bias.to(DEV),
-                       state[:, :H * d * vd], step_rows(lengths, slots), out, H, G, d, vd, a.to(DEV))
+                       state[:, :H * d * vd], step_rows(lengths, slots), out, H, G, d, vd, decays)
         at = 0
         for i, length in enumerate(lengths):
             r = slice(at, at + length)
@@ -417,6 +419,8 @@ def test_a_key_written_once_is_read_back_much_later():
     H, d, vd, n = 1, 32, 16, 300
     state = torch.zeros(1, d * vd, dtype=torch.float32, device=DEV)
     a_log, dt_bias = torch.zeros(1), torch.full((d,), -12.0)  # softplus(-12) = 6e-6: the decay is 1 - 6e-6
+    decays = torch.zeros(1, d, device=DEV)
+    ops.channel_decays(decays, a_log.to(DEV), dt_bias.to(DEV), 1, d)
     first = torch.zeros(d)
     first[0] = 1.0
     value = rnd((vd,), 5)
@@ -426,7 +430,7 @@ def test_a_key_written_once_is_read_back_much_later():
         b = torch.tensor([[20.0 if t == 0 else (-20.0 if t == n - 1 else 0.0)]])  # the last token writes nothing
         out = torch.empty(1, 1, vd, dtype=torch.float32, device=DEV)
         ops.delta_rule(key[None].to(DEV), key[None].to(DEV), v[None].to(DEV), b.to(DEV), a_log.to(DEV), dt_bias.to(DEV),
-                       state, step_rows([1], [0]), out, H, 1, d, vd, torch.zeros(1, d, device=DEV))
+                       state, step_rows([1], [0]), out, H, 1, d, vd, decays)
     want = value.double() * d ** -0.5
     assert float((out.cpu().double().flatten() - want).abs().max()) <= 5e-3 * float(want.abs().max())
 
@@ -452,13 +456,17 @@ def plain_memory(q, k, v, gates, bias, cap, S, nvec, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,d,vd,cap", [(2, 12, 20, 8.0), (1, 20, 7, 3.0), (2, 64, 48, 12.0), (1, 128, 16, 30.0), (3, 32, 33, 1.0)])
+@pytest.mark.parametrize("H,d,vd,cap", [(2, 12, 20, 8.0), (1, 20, 7, 3.0), (2, 64, 48, 12.0), (1, 128, 16, 30.0), (3, 32, 33, 1.0),
+                                        (2, 128, 128, 15.0)])
 def test_matrix_memory_over_steps_and_slots(H, d, vd, cap, dtype):
+    """Three requests in slots that are not in order: unequal portions (several chunks of the recurrence, more than
+    one round of the gates' scan, a chunk's edge, one row), single rows, two rows: read-outs and the state that is left
+    against the float64 loop over the rows.  The division rides on the norm's kernel and is checked through it."""
     from inferx_amd import ops
-    steps = [(33, 16, 1), (1, 1, 1), (1, 1, 1), (2, 17, 5), (70, 1, 31)]
+    steps = [(33, 16, 1), (1, 1, 1), (1, 1, 1), (2, 17, 5), (70, 1, 31), (130, 64, 65)]
     slots = [4, 0, 2]
     floats = ops.matrix_memory_state_floats(H, d, vd)
-    assert floats == H * d * vd + -(-vd // 16) * (H * d + H)
+    assert floats == H * d * (vd + 1) + H
     state = torch.zeros(6, floats + 3, dtype=torch.float32, device=DEV)
     state[1] = float("nan")
     own = [(torch.zeros(H, d, vd, dtype=F), torch.zeros(H, d, dtype=F), torch.zeros(H, dtype=F)) for _ in slots]
@@ -468,24 +476,29 @@ def test_matrix_memory_over_steps_and_slots(H, d, vd, cap, dtype):
         T = sum(lengths)
         q, k, v = rnd((T, H * d), 100 + n, 1.0, dtype), rnd((T, H * d), 200 + n, 1.0, dtype), rnd((T, H * vd), 300 + n, 1.0, dtype)
         gates = rnd((T, 2 * H), 400 + n, 3.0)
-        out = torch.empty(T, H, vd, dtype=torch.float32, device=DEV)
+        out, nq = torch.empty(T, H, vd, dtype=torch.float32, device=DEV), torch.empty(T, H, dtype=torch.float32, device=DEV)
+        work = torch.empty(T, H, 3, dtype=torch.float32, device=DEV)
         ops.matrix_memory(q.to(DEV), k.to(DEV), v.to(DEV), gates.to(DEV), bias.to(DEV), cap, state[:, :floats],
-                          step_rows(lengths, slots), out, H, d, vd)
+                          step_rows(lengths, slots), out, nq, work, H, d, vd)
+        read = out / (torch.maximum(nq.abs(), work[:, :, 2]) + 1e-6)[:, :, None]
+        normed = torch.empty(T, H * vd, dtype=dtype, device=DEV)
+        ops.head_norm_gate(out, normed, 1e-5, den_a=nq, den_b=work[:, :, 2])
         at = 0
         for i, length in enumerate(lengths):
             r = slice(at, at + length)
             want = plain_memory(q[r].double().view(-1, H, d), k[r].double().view(-1, H, d), v[r].double().view(-1, H, vd),
                                 gates[r].double(), bias.double(), cap, *own[i])
-            err = float((out[r].cpu().double() - want).abs().max()) / max(float(want.abs().max()), 1e-3)
+            err = float((read[r].cpu().double() - want).abs().max()) / max(float(want.abs().max()), 1e-3)
             assert err <= tol, f"step {n} request {i}: {err:.2e}"
+            unit = pg.rms_unit(want, 1e-5)
+            err = float((normed[r].cpu().double().view(-1, H, vd) - unit).abs().max()) / float(unit.abs().max())
+            assert err <= max(tol, 1e-2 if dtype == torch.bfloat16 else 0), f"step {n} request {i} normed: {err:.2e}"
             at += length
-    for i, slot in enumerate(slots):
-        S = state[slot, :H * d * vd].view(H, vd, d).transpose(1, 2).cpu().double()
+    for i, slot in enumerate(slots):  # per head [column][row] with n as the last column, then the maxima
+        matrices = state[slot, :H * d * (vd + 1)].view(H, vd + 1, d).cpu().double()
+        S, nvec = matrices[:, :vd].transpose(1, 2), matrices[:, vd]
+        top = state[slot, H * d * (vd + 1):floats].cpu().double()
         assert float((S - own[i][0]).abs().max()) <= tol * max(float(own[i][0].abs().max()), 1e-3)
-        for block in range(-(-vd // 16)):  # every block of sixteen columns carries n and m of its own
-            at = H * d * vd + block * (H * d + H)
-            nvec = state[slot, at:at + H * d].view(H, d).cpu().double()
-            top = state[slot, at + H * d:at + H * d + H].cpu().double()
-            assert float((nvec - own[i][1]).abs().max()) <= tol * max(float(own[i][1].abs().max()), 1e-3)
-            assert float((top - own[i][2]).abs().max()) <= 1e-4 * max(float(own[i][2].abs().max()), 1.0)
+        assert float((nvec - own[i][1]).abs().max()) <= tol * max(float(own[i][1].abs().max()), 1e-3)
+        assert float((top - own[i][2]).abs().max()) <= 1e-4 * max(float(own[i][2].abs().max()), 1.0)
     assert torch.isnan(state[1]).all() and float(state[3].abs().max()) == 0.0
