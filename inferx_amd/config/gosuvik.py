@@ -46,7 +46,7 @@ def _rot(raw: Any, where: str) -> Optional[Dict[str, Any]]:
         w = where + ".scaling"
         scaling = {"factor": _number(sc, "factor", w, float)}
         if any(k in sc for k in ("original", "fast", "slow")):
-            scaling.update(original=_number(sc, "original", w, int), fast=_number(sc, "fast", w, float),
+            scaling.update(original=_number(sc, "original", w, float), fast=_number(sc, "fast", w, float),
                            slow=_number(sc, "slow", w, float))
         out["scaling"] = scaling
     return out

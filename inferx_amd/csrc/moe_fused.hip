@@ -14,8 +14,10 @@ __global__ void moe_combine_add_rmsnorm_kernel(float* __restrict__ h, const T* _
                                                const int32_t* __restrict__ dest, const float* __restrict__ topk_w,
                                                const T* __restrict__ shared, const float* __restrict__ shared_gate,
                                                const void* __restrict__ w, int w_dtype, T* __restrict__ out,
-                                               const int32_t* __restrict__ rows, int64_t width, int k, float eps,
-                                               const void* __restrict__ wd, int wd_dtype, float eps_d) {
+                                               const int32_t* __restrict__ rows, int64_t row_width, int64_t width,
+                                               int k, float eps, const void* __restrict__ wd, int wd_dtype,
+                                               float eps_d) {
+  // (`width` is what one norm runs over: the row, or one of its gridDim.y equal runs, each with its own sum)
   extern __shared__ __align__(16) float vrow[];  // [width]
   __shared__ float red[16];
   __shared__ float sw[32];
@@ -28,21 +30,24 @@ __global__ void moe_combine_add_rmsnorm_kernel(float* __restrict__ h, const T* _
   }
   __syncthreads();
   const float sg = shared ? (shared_gate ? shared_gate[row] : 1.0f) : 0.f;
-  float* hr = h + row * width;
+  const int64_t first = blockIdx.y * width;
+  float* hr = h + row * row_width + first;
+  y += first;
+  if (shared) shared += first;
   float sumsq = 0.f;
   if (wd) {  // the sum is normalised before it is added
     float sumsq_d = 0.f;
     for (int64_t c = threadIdx.x; c < width; c += blockDim.x) {
       float acc = 0.f;
-      for (int s = 0; s < k; ++s) acc += sw[s] * ix_load(y + static_cast<int64_t>(sd[s]) * width + c);
-      if (shared) acc += sg * ix_load(shared + row * width + c);
+      for (int s = 0; s < k; ++s) acc += sw[s] * ix_load(y + static_cast<int64_t>(sd[s]) * row_width + c);
+      if (shared) acc += sg * ix_load(shared + row * row_width + c);
       vrow[c] = acc;
       sumsq_d += acc * acc;
     }
     sumsq_d = ix_block_sum(sumsq_d, red);
     const float inv_d = 1.0f / sqrtf(sumsq_d / static_cast<float>(width) + eps_d);
     for (int64_t c = threadIdx.x; c < width; c += blockDim.x) {  // (every thread reads back what it wrote itself)
-      const float v = hr[c] + vrow[c] * inv_d * ix_load_rt(wd, wd_dtype, c);
+      const float v = hr[c] + vrow[c] * inv_d * ix_load_rt(wd, wd_dtype, first + c);
       if (!rows) hr[c] = v;
       vrow[c] = v;
       sumsq += v * v;
@@ -50,8 +55,8 @@ __global__ void moe_combine_add_rmsnorm_kernel(float* __restrict__ h, const T* _
   } else {
     for (int64_t c = threadIdx.x; c < width; c += blockDim.x) {
       float acc = 0.f;
-      for (int s = 0; s < k; ++s) acc += sw[s] * ix_load(y + static_cast<int64_t>(sd[s]) * width + c);
-      if (shared) acc += sg * ix_load(shared + row * width + c);
+      for (int s = 0; s < k; ++s) acc += sw[s] * ix_load(y + static_cast<int64_t>(sd[s]) * row_width + c);
+      if (shared) acc += sg * ix_load(shared + row * row_width + c);
       const float v = hr[c] + acc;
       if (!rows) hr[c] = v;
       vrow[c] = v;
@@ -60,8 +65,8 @@ __global__ void moe_combine_add_rmsnorm_kernel(float* __restrict__ h, const T* _
   }
   sumsq = ix_block_sum(sumsq, red);
   const float inv = 1.0f / sqrtf(sumsq / static_cast<float>(width) + eps);
-  T* outr = out + r * width;
-  for (int64_t c = threadIdx.x; c < width; c += blockDim.x) ix_store(outr + c, vrow[c] * inv * ix_load_rt(w, w_dtype, c));
+  T* outr = out + r * row_width + first;
+  for (int64_t c = threadIdx.x; c < width; c += blockDim.x) ix_store(outr + c, vrow[c] * inv * ix_load_rt(w, w_dtype, first + c));
 }
 
 // bfloat16 with a width that is a multiple of 4: four columns per thread (8-byte loads of the experts' rows,
@@ -79,8 +84,9 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
                                                     const uint16_t* __restrict__ shared,
                                                     const float* __restrict__ shared_gate, const void* __restrict__ w,
                                                     int w_dtype, uint16_t* __restrict__ out,
-                                                    const int32_t* __restrict__ rows, int64_t width, int k, float eps,
-                                                    const void* __restrict__ wd, int wd_dtype, float eps_d) {
+                                                    const int32_t* __restrict__ rows, int64_t row_width, int64_t width,
+                                                    int k, float eps, const void* __restrict__ wd, int wd_dtype,
+                                                    float eps_d) {
   extern __shared__ __align__(16) float vrow[];  // [width]
   __shared__ float red[16];
   __shared__ float sw[32];
@@ -93,7 +99,10 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
   }
   __syncthreads();
   const float sg = shared ? (shared_gate ? shared_gate[row] : 1.0f) : 0.f;
-  float* hr = h + row * width;
+  const int64_t first = blockIdx.y * width;
+  float* hr = h + row * row_width + first;
+  y += first;
+  if (shared) shared += first;
   float sumsq = 0.f;
   float inv_d = 1.0f;
   if (wd) {  // the sum is normalised before it is added: its sum of squares first (the sum itself is formed twice)
@@ -101,12 +110,12 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
     for (int64_t c = 4 * threadIdx.x; c < width; c += 4 * blockDim.x) {
       float acc[4] = {0.f, 0.f, 0.f, 0.f}, f[4];
       for (int s = 0; s < k; ++s) {
-        bf16x4_to_f32(*reinterpret_cast<const uint2*>(y + static_cast<int64_t>(sd[s]) * width + c), f);
+        bf16x4_to_f32(*reinterpret_cast<const uint2*>(y + static_cast<int64_t>(sd[s]) * row_width + c), f);
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] += sw[s] * f[i];
       }
       if (shared) {
-        bf16x4_to_f32(*reinterpret_cast<const uint2*>(shared + row * width + c), f);
+        bf16x4_to_f32(*reinterpret_cast<const uint2*>(shared + row * row_width + c), f);
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] += sg * f[i];
       }
@@ -119,18 +128,18 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
   for (int64_t c = 4 * threadIdx.x; c < width; c += 4 * blockDim.x) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f}, f[4];
     for (int s = 0; s < k; ++s) {
-      bf16x4_to_f32(*reinterpret_cast<const uint2*>(y + static_cast<int64_t>(sd[s]) * width + c), f);
+      bf16x4_to_f32(*reinterpret_cast<const uint2*>(y + static_cast<int64_t>(sd[s]) * row_width + c), f);
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] += sw[s] * f[i];
     }
     if (shared) {
-      bf16x4_to_f32(*reinterpret_cast<const uint2*>(shared + row * width + c), f);
+      bf16x4_to_f32(*reinterpret_cast<const uint2*>(shared + row * row_width + c), f);
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] += sg * f[i];
     }
     if (wd) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[i] *= inv_d * ix_load_rt(wd, wd_dtype, c + i);
+      for (int i = 0; i < 4; ++i) acc[i] *= inv_d * ix_load_rt(wd, wd_dtype, first + c + i);
     }
     float4 v = *reinterpret_cast<const float4*>(hr + c);
     v.x += acc[0]; v.y += acc[1]; v.z += acc[2]; v.w += acc[3];
@@ -143,14 +152,14 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
   }
   sumsq = ix_block_sum(sumsq, red);
   const float inv = 1.0f / sqrtf(sumsq / static_cast<float>(width) + eps);
-  uint16_t* outr = out + r * width;
+  uint16_t* outr = out + r * row_width + first;
   for (int64_t c = 4 * threadIdx.x; c < width; c += 4 * blockDim.x) {
     const float4 v = *reinterpret_cast<const float4*>(vrow + c);
     uint2 o;
-    o.x = ix_f32_to_bf16(v.x * inv * ix_load_rt(w, w_dtype, c)) |
-          static_cast<uint32_t>(ix_f32_to_bf16(v.y * inv * ix_load_rt(w, w_dtype, c + 1))) << 16;
-    o.y = ix_f32_to_bf16(v.z * inv * ix_load_rt(w, w_dtype, c + 2)) |
-          static_cast<uint32_t>(ix_f32_to_bf16(v.w * inv * ix_load_rt(w, w_dtype, c + 3))) << 16;
+    o.x = ix_f32_to_bf16(v.x * inv * ix_load_rt(w, w_dtype, first + c)) |
+          static_cast<uint32_t>(ix_f32_to_bf16(v.y * inv * ix_load_rt(w, w_dtype, first + c + 1))) << 16;
+    o.y = ix_f32_to_bf16(v.z * inv * ix_load_rt(w, w_dtype, first + c + 2)) |
+          static_cast<uint32_t>(ix_f32_to_bf16(v.w * inv * ix_load_rt(w, w_dtype, first + c + 3))) << 16;
     *reinterpret_cast<uint2*>(outr + c) = o;
   }
 }
@@ -158,29 +167,33 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
 extern "C" int ix_moe_combine_add_rmsnorm(void* h, const void* y, int dtype, const int32_t* dest,
                                           const float* topk_w, const void* shared, const float* shared_gate,
                                           const void* w, int w_dtype, void* out, const int32_t* rows,
-                                          int64_t n_out_rows, int64_t width, int k, float eps, const void* wd,
-                                          int wd_dtype, float eps_d, hipStream_t stream) {
-  IX_REQUIRE(n_out_rows >= 0 && width > 0, "sizes must be positive");
+                                          int64_t n_out_rows, int64_t row_width, int k, float eps, const void* wd,
+                                          int wd_dtype, float eps_d, int groups, hipStream_t stream) {
+  // `groups`: the last norm runs over that many equal runs of the row, each with its own root mean square
+  IX_REQUIRE(n_out_rows >= 0 && row_width > 0, "sizes must be positive");
+  IX_REQUIRE(groups > 0 && groups <= 65535 && row_width % groups == 0, "the groups must divide the width");
+  IX_REQUIRE(groups == 1 || wd == nullptr, "a sum with a norm of its own goes with a last norm in one group");
+  const int64_t width = row_width / groups;
   IX_REQUIRE(k > 0 && k <= 32, "top_k must be between 1 and 32");
   IX_REQUIRE(width * sizeof(float) <= 60 * 1024, "hidden width too large for the fused kernel (limit 15360)");
   IX_REQUIRE(w_dtype == IX_F32 || w_dtype == IX_BF16, "weight dtype must be float32 or bfloat16");
   if (n_out_rows == 0) return 0;
-  dim3 grid(n_out_rows), block(width >= 4096 ? 1024 : (width >= 1024 ? 512 : 256));
+  dim3 grid(n_out_rows, groups), block(width >= 4096 ? 1024 : (width >= 1024 ? 512 : 256));
   const size_t smem = width * sizeof(float);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_kernel<float>, grid, block, smem, stream, (float*)h, (const float*)y,
-                       dest, topk_w, (const float*)shared, shared_gate, w, w_dtype, (float*)out, rows, width, k, eps, wd,
-                       wd_dtype, eps_d);
+                       dest, topk_w, (const float*)shared, shared_gate, w, w_dtype, (float*)out, rows, row_width, width, k, eps,
+                       wd, wd_dtype, eps_d);
   else if (dtype == IX_BF16 && width % 4 == 0 &&
            ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(shared) |
              reinterpret_cast<uintptr_t>(out)) & 15) == 0)
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_vec4_kernel, grid, dim3(width >= 4096 ? 1024 : (width >= 2048 ? 512 : 256)),
                        smem, stream, (float*)h, (const uint16_t*)y, dest, topk_w, (const uint16_t*)shared, shared_gate, w,
-                       w_dtype, (uint16_t*)out, rows, width, k, eps, wd, wd_dtype, eps_d);
+                       w_dtype, (uint16_t*)out, rows, row_width, width, k, eps, wd, wd_dtype, eps_d);
   else if (dtype == IX_BF16)
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_kernel<bf16_t>, grid, block, smem, stream, (float*)h,
                        (const bf16_t*)y, dest, topk_w, (const bf16_t*)shared, shared_gate, w, w_dtype, (bf16_t*)out,
-                       rows, width, k, eps, wd, wd_dtype, eps_d);
+                       rows, row_width, width, k, eps, wd, wd_dtype, eps_d);
   else
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_moe_combine_add_rmsnorm");

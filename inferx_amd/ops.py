@@ -731,9 +731,10 @@ def moe_combine(y: torch.Tensor, dest: torch.Tensor, topk_w: torch.Tensor, share
 def moe_combine_add_rmsnorm(h: torch.Tensor, y: torch.Tensor, dest: torch.Tensor, topk_w: torch.Tensor,
                             shared: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor], weight: torch.Tensor,
                             out: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,
-                            sum_weight: Optional[torch.Tensor] = None, sum_eps: float = 0.0) -> None:
+                            sum_weight: Optional[torch.Tensor] = None, sum_eps: float = 0.0, groups: int = 1) -> None:
     """`moe_combine` followed by `add_rmsnorm` in one pass: h += sum; out = rmsnorm(h) * weight.  With `sum_weight`
-    the sum passes an RMS norm of its own first: h += rmsnorm(sum, sum_eps) * sum_weight."""
+    the sum passes an RMS norm of its own first: h += rmsnorm(sum, sum_eps) * sum_weight.  `groups`: the last norm
+    runs over that many equal runs of the width, each with its own root mean square."""
     T, k = topk_w.shape
     H = h.shape[1]
     _need(h.dtype == torch.float32 and h.shape[0] == T, "the residual stream is float32 [T, H]")
@@ -750,7 +751,7 @@ def moe_combine_add_rmsnorm(h: torch.Tensor, y: torch.Tensor, dest: torch.Tensor
     _call("ix_moe_combine_add_rmsnorm", _ptr(h), _ptr(y), _i32(_dt(y)), _ptr(dest), _ptr(topk_w), _ptr(shared),
           _ptr(shared_gate if shared is not None else None), _ptr(weight), _i32(_dt(weight)), _ptr(out), _ptr(rows),
           _i64(n_out), _i64(H), _i32(k), _f32(eps), _ptr(sum_weight),
-          _i32(_dt(sum_weight) if sum_weight is not None else F32), _f32(sum_eps), _stream())
+          _i32(_dt(sum_weight) if sum_weight is not None else F32), _f32(sum_eps), _i32(groups), _stream())
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:

@@ -97,6 +97,10 @@ class LazyDelta:
     def materialize(self, ctx):
         raise NotImplementedError
 
+    # True: `add_rmsnorm` also takes `groups` (the norm over that many equal runs of the width, each with its own
+    # root mean square); a norm in groups asks only those that say so
+    norms_in_groups = False
+
     def add_rmsnorm(self, ctx, h, weight, eps, rows, out) -> bool:
         """h += delta; out = rmsnorm(h) * weight.  Returns False if this case is not fused (then nothing was done)."""
         return False

@@ -291,10 +291,13 @@ class MoeSum(LazyDelta):
         ops.moe_combine(self.y, self.dest, self.topk_w, self.shared, self.gate, out)
         return out
 
-    def add_rmsnorm(self, ctx, h, weight, eps, rows, out) -> bool:
+    norms_in_groups = True  # `add_rmsnorm` takes `groups`: the norm over equal runs of the width
+
+    def add_rmsnorm(self, ctx, h, weight, eps, rows, out, groups: int = 1) -> bool:
         if self.width * 4 > 60 * 1024:
             return False
-        ops.moe_combine_add_rmsnorm(h, self.y, self.dest, self.topk_w, self.shared, self.gate, weight, out, eps, rows)
+        ops.moe_combine_add_rmsnorm(h, self.y, self.dest, self.topk_w, self.shared, self.gate, weight, out, eps, rows,
+                                    groups=groups)
         return True
 
     def add_normed_rmsnorm(self, ctx, h, sum_weight, sum_eps, weight, eps, rows, out) -> bool:

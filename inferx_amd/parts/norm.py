@@ -42,8 +42,12 @@ class RMSNorm(Norm):
         n = h.shape[0] if rows is None else rows.numel()
         out = ctx.rt.empty((n, self.width))
         if isinstance(delta, LazyDelta):
-            if self.groups == 1 and delta.add_rmsnorm(ctx, h, self.weight, self.eps, rows, out):
-                return out
+            if self.groups == 1:
+                if delta.add_rmsnorm(ctx, h, self.weight, self.eps, rows, out):
+                    return out
+            elif getattr(delta, "norms_in_groups", False):  # a sum that knows how to ride on a norm in groups
+                if delta.add_rmsnorm(ctx, h, self.weight, self.eps, rows, out, groups=self.groups):
+                    return out
             delta = delta.materialize(ctx)
         ops.add_rmsnorm(h, delta, self.weight, out, self.eps, rows, self.groups)
         return out

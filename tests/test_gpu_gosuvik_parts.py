@@ -53,6 +53,29 @@ def test_norm_in_groups(width, groups, dtype, tol):
     assert float((picked.cpu().double() - want[[4, 0, 4]]).abs().max()) <= tol * float(want.abs().max())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,groups", [(96, 2), (72, 3), (128, 4), (30, 5)])
+def test_experts_sum_rides_on_the_norm_in_groups(width, groups, dtype):
+    """The experts' weighted sum, the residual add and the norm in groups in one launch against the three one by one."""
+    from inferx_amd import ops
+    T, k = 7, 3
+    y, w = rnd((T * k + 2, width), 11, 1.0, dtype).to(DEV), (rnd((width,), 12, 0.3, dtype) + 1.0).to(DEV)
+    dest = torch.randperm(T * k + 2, generator=torch.Generator().manual_seed(3))[:T * k].to(torch.int32).to(DEV)
+    topk_w = torch.rand(T, k, generator=torch.Generator().manual_seed(4)).to(DEV)
+    for rows in (None, torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)):
+        h1, h2 = rnd((T, width), 13, 2.0).to(DEV), rnd((T, width), 13, 2.0).to(DEV)
+        n = T if rows is None else 3
+        one, three = torch.empty(n, width, dtype=dtype, device=DEV), torch.empty(n, width, dtype=dtype, device=DEV)
+        ops.moe_combine_add_rmsnorm(h1, y, dest, topk_w, None, None, w, one, 1e-5, rows, groups=groups)
+        total = torch.zeros(T, width, dtype=torch.float32, device=DEV)
+        for s in range(k):
+            total += topk_w[:, s:s + 1] * y[dest.view(T, k)[:, s].long()].float()
+        ops.add_rmsnorm(h2, total, w, three, 1e-5, rows, groups)
+        assert float((h1 - h2).abs().max()) <= 1e-5 * float(h2.abs().max())
+        tol = 1e-5 if dtype == torch.float32 else 1e-2
+        assert float((one.float() - three.float()).abs().max()) <= tol * float(three.float().abs().max())
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("width", [24, 320, 4100])
 def test_polynorm_sum_and_gate(width, dtype, tol):
