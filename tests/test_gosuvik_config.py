@@ -20,7 +20,7 @@ def test_configuration_is_read_layer_by_layer():
     assert (cfg.loop_start, cfg.loop_stop, cfg.loop_times) == (0, 2, 2) and cfg.layer_order() == [0, 1, 0, 1, 2]
     m = cfg.layers[0].mixer
     assert (m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["scale"], m["window"]) == (3, 16, 8, 24, 40, 0.2, 20)
-    assert m["rot"] == {"theta": 10000.0, "rotary_dim": 8, "scaling": {"factor": 4.0, "original": 16, "fast": 8.0, "slow": 1.0}}
+    assert m["rot"] == {"theta": 10000.0, "rotary_dim": 6, "scaling": {"factor": 4.0, "original": 16, "fast": 8.0, "slow": 1.0}}
     m = cfg.layers[1].mixer
     assert (m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]) == (4, 2, 16, 12, 3)
     m = cfg.layers[2].mixer
@@ -35,6 +35,7 @@ def test_configuration_is_read_layer_by_layer():
         (lambda c: c["layers"][0].update(type="convolution"), "not a mixer"),
         (lambda c: c["layers"][0]["mixer"].pop("kv_rank"), "kv_rank"),
         (lambda c: c["layers"][0]["mixer"]["rot"].update(dims=7), "even"),
+        (lambda c: c["layers"][0]["mixer"]["rot"].update(dims=10), "at most 8"),
         (lambda c: c["layers"][0]["mixer"]["rot"]["scaling"].pop("slow"), "slow"),
         (lambda c: c["layers"][1]["mixer"].update(kv_heads=3), "multiple of kv_heads"),
         (lambda c: c["layers"][1]["mlp"]["router"].update(top=7), "between 1 and router.experts"),

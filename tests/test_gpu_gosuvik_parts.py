@@ -196,7 +196,7 @@ def run_sink_attention(paged, lengths, contexts, H, scale, window, sink, turn, d
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
-@pytest.mark.parametrize("H,G,d,vd,page,window", [(4, 2, 16, 24, 16, 9), (3, 3, 10, 6, 8, 0), (8, 1, 64, 64, 16, 96),
+@pytest.mark.parametrize("H,G,d,vd,page,window", [(4, 2, 16, 24, 16, 9), (3, 3, 10, 6, 8, 0), (6, 1, 64, 64, 16, 80),
                                                    (2, 1, 32, 48, 48, 33), (1, 1, 8, 8, 16, 1)])
 def test_attention_with_sink_window_and_values_turned_back(H, G, d, vd, page, window, dtype, tol):
     """Unequal requests in one step: portions (one from position 0), a single token between them; then single tokens.
@@ -215,7 +215,7 @@ def test_attention_with_sink_window_and_values_turned_back(H, G, d, vd, page, wi
             assert float((got - want).abs().max()) <= tol * float(want.abs().max()), f"{lengths} sink {use_sink}"
 
 
-@pytest.mark.parametrize("H,G,d,page,window", [(4, 2, 32, 16, 9), (8, 1, 64, 16, 96), (16, 4, 128, 32, 40), (3, 3, 96, 16, 0),
+@pytest.mark.parametrize("H,G,d,page,window", [(4, 2, 32, 16, 9), (8, 2, 64, 16, 72), (16, 1, 128, 32, 40), (3, 3, 96, 16, 0),
                                                 (2, 1, 48, 48, 33)])
 def test_attention_with_sink_on_the_matrix_cores(H, G, d, page, window):
     """The wavefront-level matrix-core kernel with a sink and the result turned back (heads of a multiple of 32; of 48:
@@ -238,7 +238,7 @@ def test_attention_with_sink_on_the_matrix_cores(H, G, d, page, window):
 
 
 @pytest.mark.parametrize("mfma", [False, True])
-@pytest.mark.parametrize("window", [40, 96])
+@pytest.mark.parametrize("window", [40, 72])
 @pytest.mark.parametrize("back", [0, 1, 15, 16, 17, "in", "out", "far"])
 def test_one_key_that_stands_out_at_the_windows_edge(window, back, mfma):
     """600 keys; the queries match ONE key strongly.  The key lies `back` places behind the last query: the query's own
@@ -353,11 +353,11 @@ def run_latent(contexts, lengths, H, rank, rot, page, window, dtype, mfma, stand
 
 
 @pytest.mark.parametrize("mfma", [False, True])
-@pytest.mark.parametrize("window", [0, 1, 20, 33, 96])
+@pytest.mark.parametrize("window", [0, 1, 20, 33, 80])
 def test_latent_attention_with_a_window(mfma, window):
     contexts = [70, 33, 1, 150, 48]
     dtype = torch.bfloat16 if mfma else torch.float32
-    for H, rank, rot, page in [(3, 64, 32, 16), (16, 128, 32, 16)] if mfma else [(3, 40, 8, 16), (2, 24, 10, 8)]:
+    for H, rank, rot, page in [(3, 64, 32, 16), (16, 96, 64, 16)] if mfma else [(3, 40, 8, 16), (2, 24, 10, 8)]:
         for lengths in ([70, 20, 1, 9, 16], [1, 1, 1, 1, 1], [3, 1, 1, 2, 1]):
             got, want, _ = run_latent(contexts, lengths, H, rank, rot, page, window, dtype, mfma)
             assert torch.isfinite(got).all()
@@ -366,11 +366,11 @@ def test_latent_attention_with_a_window(mfma, window):
 
 
 @pytest.mark.parametrize("mfma", [False, True])
-@pytest.mark.parametrize("distance", [0, 1, 31, 32, 63, 64, 95, 96, 97, 500])
+@pytest.mark.parametrize("distance", [0, 1, 31, 32, 63, 64, 79, 80, 81, 500])
 def test_latent_key_that_stands_out_at_the_windows_edge(mfma, distance):
-    """A window of 96 over 1,000 rows; one row takes nearly all the weight if it is visible: the query's own, a round's
-    and a page's borders, the last inside the window (95), the first outside (96)."""
-    n, window = 1000, 96
+    """A window of 80 over 1,000 rows; one row takes nearly all the weight if it is visible: the query's own, a round's
+    and a page's borders, the last inside the window (79), the first outside (80)."""
+    n, window = 1000, 80
     for lengths in ([1], [40]):
         got, want, rows = run_latent([n], lengths, 4, 64, 32, 16, window, torch.bfloat16, mfma, standout=(0, n - 1 - distance))
         if distance < window:
@@ -479,7 +479,7 @@ def plain_memory(q, k, v, gates, bias, cap, S, nvec, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,d,vd,cap", [(2, 12, 20, 8.0), (1, 20, 7, 3.0), (2, 64, 48, 12.0), (1, 128, 16, 30.0), (3, 32, 33, 1.0),
+@pytest.mark.parametrize("H,d,vd,cap", [(2, 12, 20, 8.0), (1, 20, 7, 3.0), (2, 64, 40, 10.0), (1, 128, 16, 30.0), (3, 32, 33, 1.0),
                                         (2, 128, 128, 15.0)])
 def test_matrix_memory_over_steps_and_slots(H, d, vd, cap, dtype):
     """Three requests in slots that are not in order: unequal portions (several chunks of the recurrence, more than

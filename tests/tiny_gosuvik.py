@@ -61,9 +61,10 @@ def config(vocab, width, eps, groups, layers, loop=None):
 
 
 # A: all three mixers, the first two run twice, two groups in the norm, windows shorter than the prompts, grouped
-# query heads in the delta layer and in the attention, values wider than keys, stretched rotations of both kinds
+# query heads in the delta layer and in the attention, values wider than keys, stretched rotations of both kinds, a
+# rotation of fewer dimensions than the rotated part holds
 A = config(320, 96, 1e-5, 2, [
-    latent(3, 16, 8, 24, 40, 0.2, 20, rot(8, 10000.0, yarn(4.0, 16, 8.0, 1.0)), dense(64)),
+    latent(3, 16, 8, 24, 40, 0.2, 20, rot(6, 10000.0, yarn(4.0, 16, 8.0, 1.0)), dense(64)),
     delta(4, 2, 16, 12, 3, experts(32, 6, 2)),
     pair((4, 2, 16, 24, 0.3, 9, rot(8, 100.0, {"factor": 2.0})), (2, 12, 20, 8.0), 0.7, 1.2, experts(32, 6, 2)),
 ], loop=(0, 2, 2))
