@@ -38,7 +38,8 @@ class PagedAttention(Mixer):
                  value_position: Optional[PartSpec] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
-        if head_dim % 2 or head_dim > 256:
+        general = qk_norm or value_position is not None or (value_dim is not None and int(value_dim) != int(head_dim))
+        if head_dim > 256 or (head_dim % 2 and not general):  # (the step after the product for plain heads pairs elements)
             raise ValueError(f"head_dim {head_dim} must be even and at most 256")
         self.out_bias = bool(out_bias)
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
