@@ -19,7 +19,7 @@ from test_gpu_bibevik import ChosenExperts
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LENGTHS = {"A": (5, 9, 27, 70), "B": (7, 23, 40, 75), "C": (1, 2, 33, 70), "D": (3, 50, 90)}
+LENGTHS = {"A": (5, 9, 27, 70), "B": (7, 23, 40, 75), "C": (1, 2, 33, 70), "D": (3, 50, 90), "E": (4, 19, 45)}
 # relative to the largest |logit| of the expected rows; fixed before the first run
 TOL = {"float32": ru.FP32_TOL, "bfloat16": ru.BF16_TOL}
 NAMES = sorted(tg.CONFIGS)

@@ -91,7 +91,14 @@ D = config(256, 128, 1e-5, 4, [
     delta(1, 1, 128, 32, 4, None),
     delta(4, 4, 32, 16, 2, dense(64)),
 ], loop=(1, 2, 2))
-CONFIGS = {"A": A, "B": B, "C": C, "D": D}
+# E: a width, a vocabulary and heads that are no multiple of 4 or 8 (groups of 30 numbers in the norm), short windows,
+# the pair first, a loop over the whole model
+E = config(77, 90, 1e-5, 3, [
+    pair((2, 1, 12, 14, 0.3, 5, rot(4, 200.0, {"factor": 1.5})), (3, 10, 6, 2.0), 0.5, 1.5, experts(28, 3, 1)),
+    delta(2, 1, 24, 10, 2, dense(50)),
+    latent(2, 10, 6, 14, 22, 0.25, 7, rot(6, 300.0, yarn(2.0, 8, 4.0, 0.5)), experts(28, 3, 2)),
+], loop=(0, 3, 2))
+CONFIGS = {"A": A, "B": B, "C": C, "D": D, "E": E}
 
 
 def make_folder(raw_config: dict, seed: int, out_dir: str, dtype: str = "bfloat16") -> str:
